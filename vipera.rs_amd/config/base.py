@@ -41,7 +41,8 @@ class LayerSpec:
     prefix under which the layer's weights are stored.  ``extras`` holds further
     parts by a role name for arrangements that have more than these five (norms
     after the mixer and the feed-forward, say); a block kind defines which roles
-    it reads and of which family (norm, mixer, ...) each is.
+    it reads and of which family (norm, mixer, ...) each is.  ``params`` holds constants of the arrangement itself
+    (``residual_mult``: what the sublayers' sum is multiplied by before it joins the stream).
     """
 
     block: str
@@ -52,6 +53,7 @@ class LayerSpec:
     position: PartSpec
     prefix: str
     extras: Dict[str, PartSpec] = field(default_factory=dict)
+    params: Dict[str, Any] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

@@ -739,6 +739,79 @@ extern "C" int vk_whole_norm_pack(const float* proj, long long ldp, const float*
   return 0;
 }
 
+// Queries and keys normed head by head, values optionally blended with another layer's, and all three laid out as the
+// attention kernels read them.
+//   proj [T, ldp] 32-bit: q (heads * dim) | k (kv_heads * dim) | v (kv_heads * vdim) from column 0 on
+//   q[h] <- q[h] / rms(q[h]) * q_weight over the head's dim numbers, k likewise (weights [dim], shared by the heads;
+//   null: no norm);  v <- (1 - mix) v + mix first, with `first` [T, ldf] 32-bit and `mix` one number on the device
+//   (first null: v as it is)
+//   qkv  [T, (heads + 2 kv_heads) * W]: every head padded with zeros to W >= max(dim, vdim)
+// One wave per (token, head of q, k or v).
+template <typename TO>
+__global__ __launch_bounds__(256) void head_norm_pack_kernel(const float* __restrict__ proj, long long ldp,
+                                                             const float* __restrict__ q_weight,
+                                                             const float* __restrict__ k_weight, float eps,
+                                                             const float* __restrict__ first, long long ldf,
+                                                             const float* __restrict__ mix, int heads, int kv_heads,
+                                                             int dim, int vdim, int W, long long units,
+                                                             TO* __restrict__ qkv) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const long long unit = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  if (unit >= units) return;
+  const int all = heads + 2 * kv_heads;
+  const long long t = unit / all;
+  const int h = (int)(unit % all);
+  const float* src = proj + t * ldp;
+  TO* dst = qkv + unit * W;
+  if (h < heads + kv_heads) {
+    const float* x = src + (long long)h * dim;          // q heads and k heads lie one behind the other
+    const float* weight = h < heads ? q_weight : k_weight;
+    float inv = 1.f;
+    if (weight) {
+      float ss = 0.f;
+      for (int d = lane; d < dim; d += WAVE) ss = fmaf(x[d], x[d], ss);
+      inv = 1.0f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    }
+    for (int d = lane; d < W; d += WAVE) {
+      float y = 0.f;
+      if (d < dim) y = weight ? x[d] * inv * weight[d] : x[d];
+      dst[d] = from_float<TO>(y);
+    }
+  } else {
+    const int g = h - heads - kv_heads;
+    const float* x = src + (long long)(heads + kv_heads) * dim + (long long)g * vdim;
+    const float lam = first ? mix[0] : 0.f;
+    for (int d = lane; d < W; d += WAVE) {
+      float y = 0.f;
+      if (d < vdim) {
+        y = x[d];
+        if (first) y = fmaf(lam, first[t * ldf + (long long)g * vdim + d], (1.0f - lam) * y);
+      }
+      dst[d] = from_float<TO>(y);
+    }
+  }
+}
+
+extern "C" int vk_head_norm_pack(const float* proj, long long ldp, const float* q_weight, const float* k_weight, float eps,
+                                 const float* first, long long ldf, const float* mix, int num_tokens, int heads,
+                                 int kv_heads, int dim, int vdim, int W, void* qkv, int dtype, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads < 1 || kv_heads < 1 || dim < 1 || vdim < 1 || W < dim || W < vdim || (first && !mix)) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  const long long units = (long long)num_tokens * (heads + 2 * kv_heads);
+  const unsigned blocks = (unsigned)((units + 3) / 4);
+  if (dtype == DT_F32)
+    head_norm_pack_kernel<float><<<blocks, 256, 0, s>>>(proj, ldp, q_weight, k_weight, eps, first, ldf, mix, heads,
+                                                        kv_heads, dim, vdim, W, units, (float*)qkv);
+  else if (dtype == DT_BF16)
+    head_norm_pack_kernel<bf16_t><<<blocks, 256, 0, s>>>(proj, ldp, q_weight, k_weight, eps, first, ldf, mix, heads,
+                                                         kv_heads, dim, vdim, W, units, (bf16_t*)qkv);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
 // The attention's output taken out of its padded heads and gated:
 //   out[t, h * vdim + d] = attn[t, h * W + d] * gate(g[t, h * vdim + d]);  gate_act as in vk_activation, g null: none
 template <typename T>

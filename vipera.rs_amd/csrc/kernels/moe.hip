@@ -17,8 +17,9 @@ constexpr int MOE_TILE = 64;      // places per tile of the 32-bit products; the
 // Lane l looks after experts l, l + 64, ...; a bit per expert of its own says which are taken (E <= 4096).
 //
 // `groups` > 1: the experts form that many equal groups of neighbours, a group's score is its largest logit, and
-// only experts of the `keep` best groups (the lowest group among equals) can be chosen.  `all_scores`: the weights are
-// the chosen experts' shares of the softmax over all E logits, which do not add up to one.
+// only experts of the `keep` best groups (the lowest group among equals) can be chosen.  `all_scores` 1: the weights are
+// the chosen experts' shares of the softmax over all E logits, which do not add up to one; 2: the sigmoid of each chosen
+// expert's own logit, not renormalized.
 struct Routing {
   int groups, keep, all_scores;
 };
@@ -53,7 +54,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
       if (!((kept >> (e / size)) & 1ull)) taken |= 1ull << i;
   }
   float whole_max = -INFINITY, whole_sum = 1.f;
-  if (how.all_scores) {
+  if (how.all_scores == 1) {
     for (int e = lane; e < experts; e += WAVE) whole_max = fmaxf(whole_max, z[e]);
     whole_max = wave_max(whole_max);
     float part = 0.f;
@@ -82,12 +83,12 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     }
     if ((arg & (WAVE - 1)) == lane) taken |= 1ull << (arg / WAVE);
     if (j == 0) first = best;
-    const float p = how.all_scores ? expf(best - whole_max) : expf(best - first);
+    const float p = how.all_scores == 2 ? 1.0f / (1.0f + expf(-best)) : how.all_scores ? expf(best - whole_max) : expf(best - first);
     sum += p;
     if (lane == j) mine = p;
     if (lane == 0) ids[(long long)t * top + j] = arg;
   }
-  if (lane < top) weights[(long long)t * top + lane] = mine / (how.all_scores ? whole_sum : sum);
+  if (lane < top) weights[(long long)t * top + lane] = how.all_scores == 2 ? mine : mine / (how.all_scores ? whole_sum : sum);
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
@@ -158,7 +159,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
                                                           const int* __restrict__ offsets,
                                                           const int* __restrict__ order, const int* __restrict__ tiles,
                                                           const int* __restrict__ num_tiles, int top, int width, int ff,
-                                                          float limit, float alpha, T* __restrict__ act) {
+                                                          float limit, float alpha, const float* __restrict__ in_weights,
+                                                          T* __restrict__ act) {
   if ((int)blockIdx.x >= num_tiles[0]) return;
   __shared__ float As[16][MOE_TILE + 4];
   __shared__ float Gs[16][MOE_TILE + 4];
@@ -206,11 +208,12 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
   for (int i = 0; i < 4; ++i) {
     const int r = ty * 4 + i;
     if (r >= count) continue;
+    const float w = in_weights ? in_weights[order[first + r]] : 1.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= ff) continue;
-      act[(long long)(first + r) * ff + n] = from_float<T>(expert_act(ga[i][j], ua[i][j], limit, alpha));
+      act[(long long)(first + r) * ff + n] = from_float<T>(expert_act(w * ga[i][j], w * ua[i][j], limit, alpha));
     }
   }
 }
@@ -275,6 +278,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_mma_kernel(const __bf16* __re
                                                               const int* __restrict__ tiles,
                                                               const int* __restrict__ num_tiles, int top, int width,
                                                               int ff, float limit, float alpha,
+                                                              const float* __restrict__ in_weights,
                                                               __bf16* __restrict__ act) {
   if ((int)blockIdx.x >= num_tiles[0]) return;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -301,13 +305,14 @@ __global__ __launch_bounds__(256) void moe_gate_up_mma_kernel(const __bf16* __re
   for (int tm = 0; tm < 4; ++tm) {
     const int r = wm * 64 + tm * 16 + lr;
     if (r >= count) continue;
+    const float w = in_weights ? in_weights[order[first + r]] : 1.f;
 #pragma unroll
     for (int tn = 0; tn < 2; ++tn)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int col = n0 + wn * 32 + tn * 16 + lg * 4 + i;
         if (col >= ff) continue;
-        act[(long long)(first + r) * ff + col] = (__bf16)expert_act(acc[tn][tm][i], acc[tn + 2][tm][i], limit, alpha);
+        act[(long long)(first + r) * ff + col] = (__bf16)expert_act(w * acc[tn][tm][i], w * acc[tn + 2][tm][i], limit, alpha);
       }
   }
 }
@@ -345,7 +350,7 @@ __global__ __launch_bounds__(256) void moe_down_mma_kernel(const __bf16* __restr
   }
 }
 
-// residual[t, :] (+)= sum_j weights[t, j] * pair_out[t * top + j, :], j ascending.
+// residual[t, :] (+)= sum_j weights[t, j] * pair_out[t * top + j, :], j ascending (weights null: every weight is 1).
 __global__ void moe_combine_kernel(const float* __restrict__ pair_out, const float* __restrict__ weights, int top,
                                    int width, long long total, float* __restrict__ residual, int accumulate) {
   const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -353,7 +358,7 @@ __global__ void moe_combine_kernel(const float* __restrict__ pair_out, const flo
   const long long t = idx / width;
   const int c = (int)(idx % width);
   float sum = 0.f;
-  for (int j = 0; j < top; ++j) sum = fmaf(weights[t * top + j], pair_out[(t * top + j) * width + c], sum);
+  for (int j = 0; j < top; ++j) sum = fmaf(weights ? weights[t * top + j] : 1.f, pair_out[(t * top + j) * width + c], sum);
   residual[idx] = accumulate ? residual[idx] + sum : sum;
 }
 
@@ -378,7 +383,8 @@ extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, i
   if (groups < 1 || keep < 1 || keep > groups || experts % groups != 0) return VK_BAD_ARGUMENT;
   if (groups > WAVE) return VK_UNSUPPORTED_SIZE;
   if (keep < groups && (long long)keep * (experts / groups) < top) return VK_BAD_ARGUMENT;
-  const Routing how{groups, keep, all_scores ? 1 : 0};
+  if (all_scores < 0 || all_scores > 2) return VK_BAD_ARGUMENT;
+  const Routing how{groups, keep, all_scores};
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
@@ -403,13 +409,17 @@ extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_t
                               num_tiles, stream);
 }
 
-// accumulate 0: the weighted sums are written to `residual` instead of added to it.
-extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
-                                   const int* offsets, const int* order, const int* tiles, const int* num_tiles,
-                                   const float* weights, int num_tokens, int experts, int top, int width, int ff,
-                                   float limit, float alpha, void* act, float* pair_out, float* residual,
-                                   int accumulate, void* stream) {
+// accumulate 0: the weighted sums are written to `residual` instead of added to it.  weigh_input: a pair's weight
+// multiplies what its expert reads (w h, applied to the gate and up sums, which are linear in h) instead of what it
+// returns.
+extern "C" int vk_moe_experts_weighed(const void* h, long long ldh, const void* wg, const void* wu, const void* wd,
+                                      int dtype, const int* offsets, const int* order, const int* tiles,
+                                      const int* num_tiles, const float* weights, int num_tokens, int experts, int top,
+                                      int width, int ff, float limit, float alpha, void* act, float* pair_out,
+                                      float* residual, int accumulate, int weigh_input, void* stream) {
   if (num_tokens <= 0) return 0;
+  const float* in_weights = weigh_input ? weights : nullptr;
+  const float* out_weights = weigh_input ? nullptr : weights;
   if (experts < 1 || top < 1 || width < 1 || ff < 1) return VK_BAD_ARGUMENT;
   const int pairs = num_tokens * top;
   hipStream_t s = (hipStream_t)stream;
@@ -427,13 +437,13 @@ extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg,
     }
     moe_gate_up_mma_kernel<<<up, 256, GT_LDS_BYTES, s>>>((const __bf16*)h, ldh, (const __bf16*)wg, (const __bf16*)wu,
                                                         offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
-                                                        (__bf16*)act);
+                                                        in_weights, (__bf16*)act);
     VK_LAUNCH_CHECK();
     moe_down_mma_kernel<<<down, 256, GT_LDS_BYTES, s>>>((const __bf16*)act, (const __bf16*)wd, offsets, order, tiles,
                                                         num_tiles, width, ff, pair_out);
     VK_LAUNCH_CHECK();
     const long long all = (long long)num_tokens * width;
-    moe_combine_kernel<<<(unsigned)((all + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, all, residual, accumulate);
+    moe_combine_kernel<<<(unsigned)((all + 255) / 256), 256, 0, s>>>(pair_out, out_weights, top, width, all, residual, accumulate);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -443,14 +453,14 @@ extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg,
   if (dtype == DT_F32) {
     moe_gate_up_kernel<float><<<up_grid, 256, 0, s>>>((const float*)h, ldh, (const float*)wg, (const float*)wu,
                                                       offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
-                                                      (float*)act);
+                                                      in_weights, (float*)act);
     VK_LAUNCH_CHECK();
     moe_down_kernel<float><<<down_grid, 256, 0, s>>>((const float*)act, (const float*)wd, offsets, order, tiles,
                                                      num_tiles, width, ff, pair_out);
   } else if (dtype == DT_BF16) {
     moe_gate_up_kernel<bf16_t><<<up_grid, 256, 0, s>>>((const bf16_t*)h, ldh, (const bf16_t*)wg, (const bf16_t*)wu,
                                                        offsets, order, tiles, num_tiles, top, width, ff, limit, alpha,
-                                                       (bf16_t*)act);
+                                                       in_weights, (bf16_t*)act);
     VK_LAUNCH_CHECK();
     moe_down_kernel<bf16_t><<<down_grid, 256, 0, s>>>((const bf16_t*)act, (const bf16_t*)wd, offsets, order, tiles,
                                                       num_tiles, width, ff, pair_out);
@@ -459,9 +469,18 @@ extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg,
   }
   VK_LAUNCH_CHECK();
   const long long total = (long long)num_tokens * width;
-  moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(pair_out, weights, top, width, total, residual, accumulate);
+  moe_combine_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(pair_out, out_weights, top, width, total, residual, accumulate);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_moe_experts_into(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,
+                                   const int* offsets, const int* order, const int* tiles, const int* num_tiles,
+                                   const float* weights, int num_tokens, int experts, int top, int width, int ff,
+                                   float limit, float alpha, void* act, float* pair_out, float* residual,
+                                   int accumulate, void* stream) {
+  return vk_moe_experts_weighed(h, ldh, wg, wu, wd, dtype, offsets, order, tiles, num_tiles, weights, num_tokens, experts,
+                                top, width, ff, limit, alpha, act, pair_out, residual, accumulate, 0, stream);
 }
 
 extern "C" int vk_moe_experts(const void* h, long long ldh, const void* wg, const void* wu, const void* wd, int dtype,

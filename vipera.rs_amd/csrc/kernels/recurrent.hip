@@ -19,7 +19,8 @@ __device__ __forceinline__ float softplus_f(float z) { return z > 20.0f ? z : lo
 //   conv  [C, taps] 32-bit, the last column is the current token's
 //   state row: `(taps - 1) * C` floats from `conv_offset` on, the inputs of the last taps - 1 tokens, oldest first
 //   ba    columns `b_col + h` and `a_col + h` of proj hold the projections for beta and the decay's step
-// Outputs (32-bit): qkv [T, C] (q unit * dim^-1/2, k unit, v), beta [T, heads], decay [T, heads].
+// Outputs (32-bit): qkv [T, ldq >= C] (q unit * dim^-1/2, k unit, v), beta [T, heads], decay [T, heads] (a_col < 0:
+// the decay is the caller's business, see channel_decay_kernel).
 // Grid (tokens, segments): a segment is one q or k head (its unit norm needs the whole head) or up to 1,024 value
 // channels.  No load sits behind a branch: where an input comes from (the step, the state, nowhere) picks an
 // address, and the value is masked.
@@ -39,7 +40,8 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
     const float* __restrict__ state, long long state_stride, long long conv_offset, const int* __restrict__ entry_of,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots,
     const float* __restrict__ a_log, const float* __restrict__ dt_bias, int kv_heads, int dim, int heads, int vdim,
-    int b_col, int a_col, float unit_eps, float* __restrict__ qkv, float* __restrict__ beta, float* __restrict__ decay) {
+    int b_col, int a_col, float unit_eps, float* __restrict__ qkv, long long ldq, float* __restrict__ beta,
+    float* __restrict__ decay) {
   __shared__ float scratch[16];
   const int t = blockIdx.x, seg = blockIdx.y;
   const int e = entry_of[t];
@@ -48,7 +50,7 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
   const int unit_heads = 2 * kv_heads;
   const int C = unit_heads * dim + heads * vdim;
   const float* old = state + (long long)slots[e] * state_stride + conv_offset;
-  float* out = qkv + (long long)t * C;
+  float* out = qkv + (long long)t * ldq;
   const bool unit = seg < unit_heads;
   const int first = unit ? seg * dim : unit_heads * dim + (seg - unit_heads) * PREP_SPAN;
   const int last = unit ? first + dim : min(C, first + PREP_SPAN);
@@ -82,7 +84,7 @@ __global__ __launch_bounds__(256) void delta_prepare_kernel(
     for (int h = threadIdx.x; h < heads; h += blockDim.x) {
       const float* p = proj + (long long)t * ldp;
       beta[(long long)t * heads + h] = sigmoid_f(p[b_col + h]);
-      decay[(long long)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(p[a_col + h] + dt_bias[h]));
+      if (a_col >= 0) decay[(long long)t * heads + h] = expf(-expf(a_log[h]) * softplus_f(p[a_col + h] + dt_bias[h]));
     }
 }
 
@@ -142,21 +144,23 @@ __device__ __forceinline__ float row_sum16(float v) {
 }
 
 // Gated delta rule.  Per head, with S [dim, vdim]:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q.
-// Grid (entries, heads, ceil(vdim / 16)).  An LDS row of a token: [q: 16R | k: 16R | v: 16 | beta, decay].
-template <int R, int BLOCK>
+// Grid (entries, heads, ceil(vdim / 16)).  An LDS row of a token: [q: 16R | k: 16R | (CH: g: 16R) | v: 16 | beta, decay].
+// CH: one decay per head and key channel, which scales that row of S; it lies in the token's qkv row from column
+// g_col on, [heads, dim].  `ldq` is the row stride of qkv.
+template <int R, int BLOCK, bool CH>
 __global__ __launch_bounds__(256) void delta_rule_kernel(
-    const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
-    float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
-    const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
-    float* __restrict__ out) {
-  constexpr int DP = 16 * R, ROW = 2 * DP + REC_COLS + 2, COUNT = BLOCK * ROW, LOADS = (COUNT + 255) / 256;
+    const float* __restrict__ qkv, long long ldq, int g_col, const float* __restrict__ beta,
+    const float* __restrict__ decay, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots,
+    int kv_heads, int dim, int heads, int vdim, float* __restrict__ out) {
+  constexpr int DP = 16 * R, VOFF = (CH ? 3 : 2) * DP, ROW = VOFF + REC_COLS + 2, COUNT = BLOCK * ROW;
+  constexpr int LOADS = (COUNT + 255) / 256;
   __shared__ float rows[COUNT];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane & 15, d0 = grp * R;
   const int v0 = blockIdx.z * REC_COLS, mine_col = wave * 4 + (lane >> 4), v = v0 + mine_col;
   const bool live = v < vdim;
   const int kh = h / (heads / kv_heads);
-  const int C = 2 * kv_heads * dim + heads * vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
   float* mine = state + (long long)slots[e] * state_stride + (((long long)h * gridDim.z * REC_COLS + v) * 16 + grp) * R;
   const bool fresh = entry_first[e] == 0;
@@ -172,13 +176,15 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
       // one load per element and no branch around it (a load inside a branch would be waited for there, and a
       // block's loads would arrive one after the other): the address is chosen by selects, a clamped one where
       // the element does not exist, and the value is masked afterwards
-      const bool is_q = col < DP, is_k = !is_q && col < 2 * DP, is_v = !is_q && !is_k && col < 2 * DP + REC_COLS;
-      const bool is_b = col == 2 * DP + REC_COLS;
-      const int d = is_q ? col : col - DP, c = col - 2 * DP;
-      const bool ok = x < COUNT && t < end && (is_q || is_k ? d < dim : is_v ? v0 + c < vdim : true);
+      const bool is_q = col < DP, is_k = !is_q && col < 2 * DP, is_g = CH && !is_q && !is_k && col < VOFF;
+      const bool is_v = col >= VOFF && col < VOFF + REC_COLS;
+      const bool is_b = col == VOFF + REC_COLS;
+      const int d = is_q ? col : is_k ? col - DP : col - 2 * DP, c = col - VOFF;
+      const bool ok = x < COUNT && t < end && (is_q || is_k || is_g ? d < dim : is_v ? v0 + c < vdim : (is_b || !CH));
       const long long tt = ok ? t : start;
-      const float* base = (is_q || is_k || is_v) ? qkv + tt * C : (is_b ? beta : decay) + tt * heads + h;
-      const int within = is_q ? kh * dim + d : is_k ? (kv_heads + kh) * dim + d : is_v ? 2 * kv_heads * dim + h * vdim + v0 + c : 0;
+      const float* base = (is_q || is_k || is_g || is_v) ? qkv + tt * ldq : ((is_b || CH) ? beta : decay) + tt * heads + h;
+      const int within = is_q ? kh * dim + d : is_k ? (kv_heads + kh) * dim + d : is_g ? g_col + h * dim + d
+                         : is_v ? 2 * kv_heads * dim + h * vdim + v0 + c : 0;
       const float loaded = base[ok ? within : 0];
       const float value = ok ? loaded : 0.f;
       held[i] = value;
@@ -194,30 +200,32 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(
     if (t0 + BLOCK < end) fetch(t0 + BLOCK);
     const int count = min(BLOCK, end - t0);
     // a token's numbers are read from LDS while the token before it is worked on
-    float kk[R], qq[R], b, g, val;
+    float kk[R], qq[R], gg[CH ? R : 1], b, g, val;
     auto read = [&](int j) {
       const float* row = rows + j * ROW;
-      b = row[2 * DP + REC_COLS], g = row[2 * DP + REC_COLS + 1], val = row[2 * DP + mine_col];
+      b = row[VOFF + REC_COLS], g = row[VOFF + REC_COLS + 1], val = row[VOFF + mine_col];
 #pragma unroll
       for (int i = 0; i < R; ++i) {
         kk[i] = row[DP + d0 + i];
         qq[i] = row[d0 + i];
+        if (CH) gg[i] = row[2 * DP + d0 + i];
       }
     };
     read(0);
     for (int j = 0; j < count; ++j) {
-      float k_now[R], q_now[R];
+      float k_now[R], q_now[R], g_rows[CH ? R : 1];
       const float b_now = b, g_now = g, val_now = val;
 #pragma unroll
       for (int i = 0; i < R; ++i) {
         k_now[i] = kk[i];
         q_now[i] = qq[i];
+        if (CH) g_rows[i] = gg[i];
       }
       if (j + 1 < count) read(j + 1);
       float dot[2] = {0.f, 0.f};     // two chains, even and odd rows, added at the end: a fixed order
 #pragma unroll
       for (int i = 0; i < R; ++i) {
-        S[i] *= g_now;
+        S[i] *= CH ? g_rows[i] : g_now;
         dot[i & 1] = fmaf(S[i], k_now[i], dot[i & 1]);
       }
       const float u = b_now * (val_now - row_sum16(dot[0] + dot[1]));
@@ -342,13 +350,14 @@ __device__ __forceinline__ float wave_total(float v) {
 
 // A block's fetch plan: element x = tid + i * SCAN_THREADS of the block is token x / ROW, column x % ROW; `plan[i]` is
 // token * 2^24 + the column's offset inside the token's row of the source, or -1 for an element that is always zero.
-template <int Q>
+template <int Q, bool CH>
 __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
-    const float* __restrict__ qkv, const float* __restrict__ beta, const float* __restrict__ decay,
-    float* __restrict__ state, long long state_stride, const int* __restrict__ entry_start,
-    const int* __restrict__ entry_first, const int* __restrict__ slots, int kv_heads, int dim, int heads, int vdim,
-    int key_pad, int value_pad, float* __restrict__ out) {
-  constexpr int DP = 64 * Q, ROW = 2 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
+    const float* __restrict__ qkv, long long ldq, int g_col, const float* __restrict__ beta,
+    const float* __restrict__ decay, float* __restrict__ state, long long state_stride,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots,
+    int kv_heads, int dim, int heads, int vdim, int key_pad, int value_pad, float* __restrict__ out) {
+  constexpr int DP = 64 * Q, VOFF = (CH ? 3 : 2) * DP, ROW = VOFF + SCAN_COLS, COUNT = REC_BLOCK * ROW;
+  constexpr int LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
   __shared__ float rows[COUNT];
   __shared__ float gates[REC_BLOCK][2];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -356,7 +365,6 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
   const int v0 = blockIdx.z * SCAN_COLS, v = v0 + wave;
   const bool live = v < vdim;
   const int kh = h / (heads / kv_heads);
-  const int C = 2 * kv_heads * dim + heads * vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
   float* mine = state + (long long)slots[e] * state_stride + ((long long)h * value_pad + v) * key_pad + d0;
   const bool fresh = entry_first[e] == 0, kept = v < value_pad;
@@ -371,7 +379,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     if (x < COUNT) {
       if (col < DP) { if (col < dim) within = kh * dim + col; }
       else if (col < 2 * DP) { if (col - DP < dim) within = (kv_heads + kh) * dim + col - DP; }
-      else if (v0 + col - 2 * DP < vdim) within = 2 * kv_heads * dim + h * vdim + v0 + col - 2 * DP;
+      else if (CH && col < VOFF) { if (col - 2 * DP < dim) within = g_col + h * dim + col - 2 * DP; }
+      else if (v0 + col - VOFF < vdim) within = 2 * kv_heads * dim + h * vdim + v0 + col - VOFF;
     }
     plan[i] = within < 0 ? -1 : (j << 24) | within;
   }
@@ -381,12 +390,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     for (int i = 0; i < LOADS; ++i) {
       // a token past the entry's end is never worked on: its address is clamped, its value does not matter
       const int t = min(t0 + (plan[i] >> 24 & 127), end - 1);
-      const float loaded = qkv[(long long)t * C + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
+      const float loaded = qkv[(long long)t * ldq + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
       held[i] = plan[i] < 0 ? 0.f : loaded;
     }
     if (tid < 2 * REC_BLOCK) {
       const int t = min(t0 + (tid >> 1), end - 1);
-      held_gate = ((tid & 1) ? decay : beta)[(long long)t * heads + h];
+      held_gate = ((tid & 1) && !CH ? decay : beta)[(long long)t * heads + h];
     }
   };
   fetch(start);
@@ -401,7 +410,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     const int count = min(REC_BLOCK, end - t0);
     for (int j = 0; j < count; ++j) {
       const float* row = rows + j * ROW;
-      const float b = gates[j][0], g = gates[j][1], val = row[2 * DP + wave];
+      const float b = gates[j][0], g = gates[j][1], val = row[VOFF + wave];
       float kk[Q], qq[Q];
 #pragma unroll
       for (int i = 0; i < Q; ++i) {
@@ -411,7 +420,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
       float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < Q; ++i) {
-        S[i] *= g;
+        S[i] *= CH ? row[2 * DP + d0 + i] : g;
         dot = fmaf(S[i], kk[i], dot);
       }
       const float u = b * (val - wave_total(dot));
@@ -553,7 +562,7 @@ __global__ __launch_bounds__(256) void save_last_kernel(const T* __restrict__ h,
 // ---------------------------------------------------------------------------------------------
 // Read-out of a recurrent head: o / rms(o) (per head, over its `vdim` channels) * weight * gate.
 // weight: [vdim] shared by the heads, or [heads * vdim]; gate: a column range of a [T, ldg] buffer of type TG,
-// passed through silu first if asked.  One wave per (token, head).
+// as it is (`gate_silu` 0), through silu (1) or through the sigmoid (2).  One wave per (token, head).
 template <typename TG, typename TO>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ weight,
                                                              int weight_per_head, const TG* __restrict__ gate,
@@ -570,10 +579,198 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
   for (int c = lane; c < vdim; c += WAVE) {
     float g = to_float<TG>(gate[(long long)t * ldg + h * vdim + c]);
-    if (gate_silu) g = silu_f(g);
+    if (gate_silu == 1) g = silu_f(g);
+    else if (gate_silu == 2) g = sigmoid_f(g);
     const float w = weight[(weight_per_head ? h * vdim : 0) + c];
     out[unit * vdim + c] = from_float<TO>(src[c] * inv * w * g);
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Matrix memory with exponential gates (mLSTM).  Per head, with S [dim, vdim], n [dim] and a running maximum m of the
+// gates' logarithms (all zero at position 0):
+//   li = cap tanh(i_raw / cap),  lf = logsigmoid(cap tanh(f_raw / cap))
+//   m' = max(lf + m, li);  a = exp(lf + m - m'),  b = exp(li - m')
+//   S <- a S + b k v^T;  n <- a n + b k;  o = S^T q / (max(|n . q|, exp(-m')) + 1e-6)
+// All operands are columns of one 32-bit buffer `proj [T, ldp]`: q (heads * dim) from q_col on, k from k_col, v
+// (heads * vdim) from v_col, the raw gates at i_col + h and f_col + h; q is multiplied by `q_scale` as it is read.
+// State row of a request: the heads' matrices in the recurrences' common layout, then n and m once per tile of eight
+// value channels ([heads][tiles][key_pad] and [heads][tiles]): every workgroup carries n and m itself, so it reads and
+// writes copies of its own and no workgroup waits for another.
+struct MemoryColumns {
+  int q, k, v, i, f;
+};
+
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+__device__ __forceinline__ float log_gate(float raw, float cap, bool forget) {
+  const float z = cap * tanhf(raw / cap);
+  return forget ? log_sigmoid_f(z) : z;
+}
+
+// Steps of single tokens: the delta rule's shape (a workgroup owns 16 value channels of one (entry, head), the sixteen
+// lanes of a row keep R key channels each of S and of n).  Grid (entries, heads, ceil(vdim / 16)).
+template <int R>
+__global__ __launch_bounds__(256) void memory_rule_kernel(
+    const float* __restrict__ proj, long long ldp, MemoryColumns col, float q_scale, float cap,
+    float* __restrict__ state, long long state_stride, long long n_offset, long long m_offset,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
+    int heads, int vdim, float* __restrict__ out) {
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane & 15, d0 = grp * R, key_pad = 16 * R;
+  const int v0 = blockIdx.z * REC_COLS, v = v0 + wave * 4 + (lane >> 4);
+  const bool live = v < vdim;
+  const int tiles = 2 * gridDim.z;       // tiles of eight value channels: this workgroup owns 2 z and 2 z + 1
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* row = state + (long long)slots[e] * state_stride;
+  float* mine = row + (((long long)h * gridDim.z * REC_COLS + v) * 16 + grp) * R;
+  float* my_n = row + n_offset + ((long long)h * tiles + 2 * blockIdx.z) * key_pad + d0;
+  float* my_m = row + m_offset + (long long)h * tiles + 2 * blockIdx.z;
+  const bool fresh = entry_first[e] == 0;
+  float S[R], N[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const float s_old = mine[i], n_old = my_n[i];
+    S[i] = fresh ? 0.f : s_old;
+    N[i] = fresh ? 0.f : n_old;
+  }
+  const float m_old = my_m[0];
+  float m = fresh ? 0.f : m_old;
+  for (int t = start; t < end; ++t) {
+    const float* p = proj + (long long)t * ldp;
+    const float li = log_gate(p[col.i + h], cap, false), lf = log_gate(p[col.f + h], cap, true);
+    const float val_loaded = p[col.v + h * vdim + (live ? v : 0)];
+    const float val = live ? val_loaded : 0.f;
+    float kk[R], qq[R];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const bool in = d0 + i < dim;
+      const float k_loaded = p[col.k + h * dim + (in ? d0 + i : 0)], q_loaded = p[col.q + h * dim + (in ? d0 + i : 0)];
+      kk[i] = in ? k_loaded : 0.f;
+      qq[i] = in ? q_loaded * q_scale : 0.f;
+    }
+    const float m_new = fmaxf(lf + m, li);
+    const float a = expf(lf + m - m_new), b = expf(li - m_new);
+    m = m_new;
+    float num[2] = {0.f, 0.f}, den[2] = {0.f, 0.f};     // two chains each, even and odd rows: a fixed order
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      const float bk = b * kk[i];
+      S[i] = fmaf(bk, val, a * S[i]);
+      N[i] = fmaf(a, N[i], bk);
+      num[i & 1] = fmaf(S[i], qq[i], num[i & 1]);
+      den[i & 1] = fmaf(N[i], qq[i], den[i & 1]);
+    }
+    const float top = row_sum16(num[0] + num[1]), under = row_sum16(den[0] + den[1]);
+    if (live && grp == 0) out[((long long)t * heads + h) * vdim + v] = top / (fmaxf(fabsf(under), expf(-m)) + 1e-6f);
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) mine[i] = S[i];
+  if (wave == 0 && lane < 16) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      my_n[i] = N[i];
+      my_n[key_pad + i] = N[i];
+    }
+    if (lane == 0) my_m[0] = my_m[1] = m;
+  }
+}
+
+// Prompts' portions: the scan shape (a wave owns one value channel and its 64 lanes the key channels, eight waves to a
+// workgroup, tokens through LDS in blocks of 16 fetched a block ahead).  Every wave carries n and m itself.
+// An LDS row of a token: [q: 64Q | k: 64Q | v: 8]; the two gates' logarithms lie beside.  Grid (entries, heads, tiles).
+template <int Q>
+__global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
+    const float* __restrict__ proj, long long ldp, MemoryColumns col, float q_scale, float cap,
+    float* __restrict__ state, long long state_stride, long long n_offset, long long m_offset,
+    const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
+    int heads, int vdim, int key_pad, int value_pad, float* __restrict__ out) {
+  constexpr int DP = 64 * Q, ROW = 2 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
+  __shared__ float rows[COUNT];
+  __shared__ float gates[REC_BLOCK][2];
+  const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int d0 = lane * Q;
+  const int v0 = blockIdx.z * SCAN_COLS, v = v0 + wave;
+  const bool live = v < vdim;
+  const int start = entry_start[e], end = entry_start[e + 1];
+  float* row0 = state + (long long)slots[e] * state_stride;
+  float* mine = row0 + ((long long)h * value_pad + v) * key_pad + d0;
+  float* my_n = row0 + n_offset + ((long long)h * gridDim.z + blockIdx.z) * key_pad + d0;
+  float* my_m = row0 + m_offset + (long long)h * gridDim.z + blockIdx.z;
+  const bool fresh = entry_first[e] == 0;
+  float S[Q], N[Q];
+#pragma unroll
+  for (int i = 0; i < Q; ++i) {
+    const bool in = d0 + i < key_pad;
+    const float s_old = mine[in ? i : -d0], n_old = my_n[in ? i : -d0];     // a clamped address where the lane has no row
+    S[i] = (!fresh && in) ? s_old : 0.f;
+    N[i] = (!fresh && in) ? n_old : 0.f;
+  }
+  const float m_old = my_m[0];
+  float m = fresh ? 0.f : m_old;
+  // a block's fetch plan: token * 2^24 + the column inside the token's row of proj, or -1 for what is always zero
+  int plan[LOADS];
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int x = tid + i * SCAN_THREADS, j = x / ROW, c = x % ROW;
+    int within = -1;
+    if (x < COUNT) {
+      if (c < DP) { if (c < dim) within = col.q + h * dim + c; }
+      else if (c < 2 * DP) { if (c - DP < dim) within = col.k + h * dim + c - DP; }
+      else if (v0 + c - 2 * DP < vdim) within = col.v + h * vdim + v0 + c - 2 * DP;
+    }
+    plan[i] = within < 0 ? -1 : (j << 24) | within;
+  }
+  float held[LOADS], held_gate = 0.f;
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const int t = min(t0 + (plan[i] >> 24 & 127), end - 1);
+      const float loaded = proj[(long long)t * ldp + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
+      const bool is_q = (tid + i * SCAN_THREADS) % ROW < DP;
+      held[i] = plan[i] < 0 ? 0.f : is_q ? loaded * q_scale : loaded;
+    }
+    if (tid < 2 * REC_BLOCK) {
+      const int t = min(t0 + (tid >> 1), end - 1);
+      held_gate = log_gate(proj[(long long)t * ldp + ((tid & 1) ? col.f : col.i) + h], cap, tid & 1);
+    }
+  };
+  fetch(start);
+  for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
+    __syncthreads();     // the block before has been read
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i)
+      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+    if (tid < 2 * REC_BLOCK) gates[tid >> 1][tid & 1] = held_gate;
+    __syncthreads();
+    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    const int count = min(REC_BLOCK, end - t0);
+    for (int j = 0; j < count; ++j) {
+      const float* row = rows + j * ROW;
+      const float li = gates[j][0], lf = gates[j][1], val = row[2 * DP + wave];
+      const float m_new = fmaxf(lf + m, li);
+      const float a = expf(lf + m - m_new), b = expf(li - m_new);
+      m = m_new;
+      float num = 0.f, den = 0.f;
+#pragma unroll
+      for (int i = 0; i < Q; ++i) {
+        const float bk = b * row[DP + d0 + i], qq = row[d0 + i];
+        S[i] = fmaf(bk, val, a * S[i]);
+        N[i] = fmaf(a, N[i], bk);
+        num = fmaf(S[i], qq, num);
+        den = fmaf(N[i], qq, den);
+      }
+      num = wave_total(num);
+      den = wave_total(den);
+      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < Q; ++i)
+    if (d0 + i < key_pad) {
+      mine[i] = S[i];
+      if (wave == 0) my_n[i] = N[i];
+    }
+  if (tid == 0) my_m[0] = m;
 }
 
 // x[t, c] = exp(-exp(x[t, c] + w0[c])) in place: time mixing's decay, for a step whose recurrence reads it many times.
@@ -591,28 +788,66 @@ __global__ void tanh_kernel(const float* __restrict__ x, TO* __restrict__ out, l
 
 // ---------------------------------------------------------------------------------------------
 
-extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* conv, int taps, float* state,
-                                long long state_stride, long long conv_offset, const int* entry_of,
-                                const int* entry_start, const int* entry_first, const int* slots, const float* a_log,
-                                const float* dt_bias, int kv_heads, int dim, int heads, int vdim, int b_col, int a_col,
-                                float unit_eps, float* qkv, float* beta, float* decay, int num_tokens, int num_entries,
-                                void* stream) {
+extern "C" int vk_delta_prepare_strided(const float* proj, long long ldp, const float* conv, int taps, float* state,
+                                        long long state_stride, long long conv_offset, const int* entry_of,
+                                        const int* entry_start, const int* entry_first, const int* slots,
+                                        const float* a_log, const float* dt_bias, int kv_heads, int dim, int heads,
+                                        int vdim, int b_col, int a_col, float unit_eps, float* qkv, long long ldq,
+                                        float* beta, float* decay, int num_tokens, int num_entries, void* stream) {
   if (num_tokens <= 0) return 0;
   if (taps < 1 || kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
   const long long C = 2LL * kv_heads * dim + (long long)heads * vdim;
   if (dim > PREP_SPAN || C > 0x7fffffff) return VK_UNSUPPORTED_SIZE;
+  if (ldq < C || (a_col >= 0 && (!decay || !a_log || !dt_bias))) return VK_BAD_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
   const long long segments = 2LL * kv_heads + ((long long)heads * vdim + PREP_SPAN - 1) / PREP_SPAN;
   if (segments > 65535) return VK_UNSUPPORTED_SIZE;
   delta_prepare_kernel<<<dim3(num_tokens, (unsigned)segments), 256, 0, s>>>(
       proj, ldp, conv, taps, state, state_stride, conv_offset, entry_of, entry_start, entry_first, slots, a_log, dt_bias,
-      kv_heads, dim, heads, vdim, b_col, a_col, unit_eps, qkv, beta, decay);
+      kv_heads, dim, heads, vdim, b_col, a_col, unit_eps, qkv, ldq, beta, decay);
   VK_LAUNCH_CHECK();
   if (taps > 1) {
     conv_state_kernel<<<dim3(num_entries, (unsigned)((C + 255) / 256)), 256, 0, s>>>(
         proj, ldp, taps, (int)C, state, state_stride, conv_offset, entry_start, entry_first, slots);
     VK_LAUNCH_CHECK();
   }
+  return 0;
+}
+
+extern "C" int vk_delta_prepare(const float* proj, long long ldp, const float* conv, int taps, float* state,
+                                long long state_stride, long long conv_offset, const int* entry_of,
+                                const int* entry_start, const int* entry_first, const int* slots, const float* a_log,
+                                const float* dt_bias, int kv_heads, int dim, int heads, int vdim, int b_col, int a_col,
+                                float unit_eps, float* qkv, float* beta, float* decay, int num_tokens, int num_entries,
+                                void* stream) {
+  if (a_col < 0) return VK_BAD_ARGUMENT;
+  return vk_delta_prepare_strided(proj, ldp, conv, taps, state, state_stride, conv_offset, entry_of, entry_start,
+                                  entry_first, slots, a_log, dt_bias, kv_heads, dim, heads, vdim, b_col, a_col, unit_eps,
+                                  qkv, 2LL * kv_heads * dim + (long long)heads * vdim, beta, decay, num_tokens,
+                                  num_entries, stream);
+}
+
+// out[t, h * dim + d] = exp(-exp(a_log[h]) * softplus(raw[t, h * dim + d] + dt_bias[h * dim + d])): the delta rule's
+// decay per head and key channel.  `raw` and `out` are 32-bit with row strides of their own.
+__global__ void channel_decay_kernel(const float* __restrict__ raw, long long ldr, const float* __restrict__ a_log,
+                                     const float* __restrict__ dt_bias, int dim, int width, long long total,
+                                     float* __restrict__ out, long long ldo) {
+  const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long long t = idx / width;
+  const int c = (int)(idx % width);
+  out[t * ldo + c] = expf(-expf(a_log[c / dim]) * softplus_f(raw[t * ldr + c] + dt_bias[c]));
+}
+
+extern "C" int vk_channel_decay(const float* raw, long long ldr, const float* a_log, const float* dt_bias, int heads,
+                                int dim, int num_tokens, float* out, long long ldo, void* stream) {
+  if (num_tokens <= 0) return 0;
+  if (heads < 1 || dim < 1) return VK_BAD_ARGUMENT;
+  const int width = heads * dim;
+  const long long total = (long long)num_tokens * width;
+  channel_decay_kernel<<<(unsigned)((total + 255) / 256), 256, 0, (hipStream_t)stream>>>(raw, ldr, a_log, dt_bias, dim,
+                                                                                        width, total, out, ldo);
+  VK_LAUNCH_CHECK();
   return 0;
 }
 
@@ -624,38 +859,107 @@ extern "C" long long vk_recurrent_head_floats(int dim, int vdim) {
   return (long long)((vdim + REC_COLS - 1) / REC_COLS) * REC_COLS * 16 * rows_of(dim);
 }
 
-extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
-                             long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
-                             int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, int short_entries,
-                             void* stream) {
+// `g_col` >= 0: one decay per head and key channel, in columns g_col.. of the qkv rows ([heads, dim]; `decay` is not
+// read); below 0: one decay per head, `decay` [T, heads].  `ldq` is the row stride of qkv.
+extern "C" int vk_delta_rule_strided(const float* qkv, long long ldq, int g_col, const float* beta, const float* decay,
+                                     float* state, long long state_stride, const int* entry_start,
+                                     const int* entry_first, const int* slots, int kv_heads, int dim, int heads, int vdim,
+                                     float* out, int num_entries, int short_entries, void* stream) {
   if (num_entries <= 0) return 0;
   if (kv_heads < 1 || heads < 1 || dim < 1 || vdim < 1 || heads % kv_heads) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535) return VK_UNSUPPORTED_SIZE;
+  const long long C = 2LL * kv_heads * dim + (long long)heads * vdim;
+  if (ldq < C || (g_col < 0 && !decay) || (g_col >= 0 && g_col + (long long)heads * dim > ldq)) return VK_BAD_ARGUMENT;
+  if (ldq >= (1 << 24)) return VK_UNSUPPORTED_SIZE;      // the prompt form keeps a column in 24 bits
   dim3 grid(num_entries, heads, (vdim + REC_COLS - 1) / REC_COLS);
   hipStream_t s = (hipStream_t)stream;
   const int key_pad = 16 * rows_of(dim), value_pad = (vdim + REC_COLS - 1) / REC_COLS * REC_COLS;
+  const bool ch = g_col >= 0;
   if (!short_entries) {
     dim3 scan_grid(num_entries, heads, value_pad / SCAN_COLS);
-#define VK_DELTA_SCAN(Q)                                                                                             \
-  delta_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start,         \
-                                                          entry_first, slots, kv_heads, dim, heads, vdim, key_pad,    \
-                                                          value_pad, out)
-    if (key_pad <= 64) VK_DELTA_SCAN(1);
-    else if (key_pad <= 128) VK_DELTA_SCAN(2);
-    else VK_DELTA_SCAN(4);
+#define VK_DELTA_SCAN(Q, CH)                                                                                         \
+  delta_scan_kernel<Q, CH><<<scan_grid, SCAN_THREADS, 0, s>>>(qkv, ldq, g_col, beta, decay, state, state_stride,       \
+                                                              entry_start, entry_first, slots, kv_heads, dim, heads,  \
+                                                              vdim, key_pad, value_pad, out)
+    if (key_pad <= 64) { if (ch) VK_DELTA_SCAN(1, true); else VK_DELTA_SCAN(1, false); }
+    else if (key_pad <= 128) { if (ch) VK_DELTA_SCAN(2, true); else VK_DELTA_SCAN(2, false); }
+    else { if (ch) VK_DELTA_SCAN(4, true); else VK_DELTA_SCAN(4, false); }
 #undef VK_DELTA_SCAN
     VK_LAUNCH_CHECK();
     return 0;
   }
-#define VK_DELTA(R)                                                                                                    \
-  delta_rule_kernel<R, 1><<<grid, 256, 0, s>>>(qkv, beta, decay, state, state_stride, entry_start, entry_first, slots, \
-                                               kv_heads, dim, heads, vdim, out)
+#define VK_DELTA(R)                                                                                                     \
+  do {                                                                                                                  \
+    if (ch)                                                                                                             \
+      delta_rule_kernel<R, 1, true><<<grid, 256, 0, s>>>(qkv, ldq, g_col, beta, decay, state, state_stride, entry_start, \
+                                                         entry_first, slots, kv_heads, dim, heads, vdim, out);          \
+    else                                                                                                                \
+      delta_rule_kernel<R, 1, false><<<grid, 256, 0, s>>>(qkv, ldq, g_col, beta, decay, state, state_stride,            \
+                                                          entry_start, entry_first, slots, kv_heads, dim, heads, vdim,  \
+                                                          out);                                                         \
+  } while (0)
   if (dim <= 16) { VK_DELTA(1); }
   else if (dim <= 32) { VK_DELTA(2); }
   else if (dim <= 64) { VK_DELTA(4); }
   else if (dim <= 128) { VK_DELTA(8); }
   else { VK_DELTA(16); }
 #undef VK_DELTA
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int vk_delta_rule(const float* qkv, const float* beta, const float* decay, float* state,
+                             long long state_stride, const int* entry_start, const int* entry_first, const int* slots,
+                             int kv_heads, int dim, int heads, int vdim, float* out, int num_entries, int short_entries,
+                             void* stream) {
+  return vk_delta_rule_strided(qkv, 2LL * kv_heads * dim + (long long)heads * vdim, -1, beta, decay, state, state_stride,
+                               entry_start, entry_first, slots, kv_heads, dim, heads, vdim, out, num_entries,
+                               short_entries, stream);
+}
+
+// Floats of one request's matrix-memory state: the heads' matrices, then n and m per tile of eight value channels.
+extern "C" long long vk_memory_state_floats(int heads, int dim, int vdim) {
+  const long long tiles = (vdim + REC_COLS - 1) / REC_COLS * (REC_COLS / SCAN_COLS);
+  return (long long)heads * (vk_recurrent_head_floats(dim, vdim) + tiles * 16 * rows_of(dim) + tiles);
+}
+
+extern "C" int vk_memory_rule(const float* proj, long long ldp, int q_col, int k_col, int v_col, int i_col, int f_col,
+                              float q_scale, float cap, float* state, long long state_stride, const int* entry_start,
+                              const int* entry_first, const int* slots, int dim, int heads, int vdim, float* out,
+                              int num_entries, int short_entries, void* stream) {
+  if (num_entries <= 0) return 0;
+  if (heads < 1 || dim < 1 || vdim < 1 || !(cap > 0.f)) return VK_BAD_ARGUMENT;
+  if (dim > 256 || heads > 65535 || ldp >= (1 << 24)) return VK_UNSUPPORTED_SIZE;
+  if (min(min(q_col, k_col), min(v_col, min(i_col, f_col))) < 0) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  const int key_pad = 16 * rows_of(dim), value_pad = (vdim + REC_COLS - 1) / REC_COLS * REC_COLS;
+  const long long tiles = value_pad / SCAN_COLS;
+  const long long n_offset = (long long)heads * vk_recurrent_head_floats(dim, vdim);
+  const long long m_offset = n_offset + (long long)heads * tiles * key_pad;
+  const MemoryColumns col{q_col, k_col, v_col, i_col, f_col};
+  if (!short_entries) {
+    dim3 scan_grid(num_entries, heads, (unsigned)tiles);
+#define VK_MEMORY_SCAN(Q)                                                                                            \
+  memory_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(proj, ldp, col, q_scale, cap, state, state_stride, n_offset, \
+                                                           m_offset, entry_start, entry_first, slots, dim, heads, vdim, \
+                                                           key_pad, value_pad, out)
+    if (key_pad <= 64) VK_MEMORY_SCAN(1);
+    else if (key_pad <= 128) VK_MEMORY_SCAN(2);
+    else VK_MEMORY_SCAN(4);
+#undef VK_MEMORY_SCAN
+    VK_LAUNCH_CHECK();
+    return 0;
+  }
+  dim3 grid(num_entries, heads, value_pad / REC_COLS);
+#define VK_MEMORY(R)                                                                                                  \
+  memory_rule_kernel<R><<<grid, 256, 0, s>>>(proj, ldp, col, q_scale, cap, state, state_stride, n_offset, m_offset,   \
+                                             entry_start, entry_first, slots, dim, heads, vdim, out)
+  if (dim <= 16) { VK_MEMORY(1); }
+  else if (dim <= 32) { VK_MEMORY(2); }
+  else if (dim <= 64) { VK_MEMORY(4); }
+  else if (dim <= 128) { VK_MEMORY(8); }
+  else { VK_MEMORY(16); }
+#undef VK_MEMORY
   VK_LAUNCH_CHECK();
   return 0;
 }

@@ -955,17 +955,20 @@ def _entries_ok(batch_arrays, num_entries: int) -> None:
 
 
 def delta_prepare(proj: torch.Tensor, conv: torch.Tensor, state: torch.Tensor, conv_offset: int, entry_of: torch.Tensor,
-                  entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, a_log: torch.Tensor,
-                  dt_bias: torch.Tensor, kv_heads: int, dim: int, heads: int, vdim: int, b_col: int, a_col: int,
-                  unit_eps: float, qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, num_entries: int) -> None:
+                  entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, a_log: Optional[torch.Tensor],
+                  dt_bias: Optional[torch.Tensor], kv_heads: int, dim: int, heads: int, vdim: int, b_col: int, a_col: int,
+                  unit_eps: float, qkv: torch.Tensor, beta: torch.Tensor, decay: Optional[torch.Tensor],
+                  num_entries: int) -> None:
     """Short causal convolution, silu, unit norms of q and k, beta and the decay for every token of the step (see
-    ``recurrent.hip``); then the convolution's state rows are replaced by the entries' last inputs."""
+    ``recurrent.hip``); then the convolution's state rows are replaced by the entries' last inputs.  ``qkv`` may be the
+    first columns of wider rows.  ``a_col`` below 0: no decay per head is computed (``a_log``, ``dt_bias`` and ``decay``
+    may be None): the caller has one per key channel, see :func:`channel_decay`."""
     _dev(proj, conv, state, entry_of, entry_start, entry_first, slots, a_log, dt_bias, qkv, beta, decay)
     tokens = proj.shape[0]
     channels = 2 * kv_heads * dim + heads * vdim
     taps = conv.shape[1]
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "delta_prepare: proj")
-    _need(proj.shape[1] >= max(channels, b_col + heads, a_col + heads) and min(b_col, a_col) >= 0, "delta_prepare: columns")
+    _need(proj.shape[1] >= max(channels, b_col + heads, a_col + heads) and b_col >= 0, "delta_prepare: columns")
     _need(conv.shape == (channels, taps) and taps >= 1, "delta_prepare: conv shape")
     _f32(conv, "delta_prepare: conv")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
@@ -973,42 +976,108 @@ def delta_prepare(proj: torch.Tensor, conv: torch.Tensor, state: torch.Tensor, c
     _i32(entry_of)
     _need(entry_of.numel() >= tokens, "delta_prepare: entry_of")
     _entries_ok((entry_start, entry_first, slots), num_entries)
-    for name, t in (("a_log", a_log), ("dt_bias", dt_bias)):
-        _need(t.dtype == torch.float32 and t.numel() == heads, f"delta_prepare: {name}")
-    _need(qkv.shape == (tokens, channels) and beta.shape == (tokens, heads) and decay.shape == (tokens, heads),
-          "delta_prepare: output shapes")
-    for t in (qkv, beta, decay):
-        _f32(t, "delta_prepare: outputs")
-    fn = _fn("recurrent", "vk_delta_prepare",
-             [_p, _ll, _p, _i, _p, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _p, _p, _p, _i, _i, _p])
+    _need(qkv.dim() == 2 and qkv.shape == (tokens, channels) and qkv.dtype == torch.float32 and qkv.stride(1) == 1
+          and qkv.stride(0) >= channels, "delta_prepare: qkv")
+    _need(beta.shape == (tokens, heads), "delta_prepare: beta")
+    _f32(beta, "delta_prepare: beta")
+    if a_col >= 0:
+        for name, t in (("a_log", a_log), ("dt_bias", dt_bias)):
+            _need(t is not None and t.dtype == torch.float32 and t.numel() == heads, f"delta_prepare: {name}")
+        _need(decay is not None and decay.shape == (tokens, heads), "delta_prepare: decay")
+        _f32(decay, "delta_prepare: decay")
+    fn = _fn("recurrent", "vk_delta_prepare_strided",
+             [_p, _ll, _p, _i, _p, _ll, _ll, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _p, _ll, _p, _p, _i, _i, _p])
     _status(fn(_ptr(proj), proj.stride(0), _ptr(conv), taps, _ptr(state), state.stride(0), conv_offset, _ptr(entry_of),
                _ptr(entry_start), _ptr(entry_first), _ptr(slots), _ptr(a_log), _ptr(dt_bias), kv_heads, dim, heads, vdim,
-               b_col, a_col, float(unit_eps), _ptr(qkv), _ptr(beta), _ptr(decay), tokens, num_entries, _stream()),
-            "delta_prepare")
+               b_col, a_col, float(unit_eps), _ptr(qkv), qkv.stride(0), _ptr(beta), _ptr(decay), tokens, num_entries,
+               _stream()), "delta_prepare")
 
 
-def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: torch.Tensor, state: torch.Tensor,
+def channel_decay(raw: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, heads: int, dim: int,
+                  out: torch.Tensor) -> None:
+    """``out[t, h, d] = exp(-exp(a_log[h]) * softplus(raw[t, h, d] + dt_bias[h, d]))``: one decay per head and key
+    channel; ``raw`` and ``out`` 32-bit ``[tokens, heads * dim]``, row-strided views are fine."""
+    _dev(raw, a_log, dt_bias, out)
+    tokens = raw.shape[0]
+    for name, t in (("raw", raw), ("out", out)):
+        _need(t.dtype == torch.float32 and t.shape == (tokens, heads * dim) and t.stride(1) == 1, f"channel_decay: {name}")
+    _need(a_log.dtype == torch.float32 and a_log.numel() == heads and a_log.is_contiguous(), "channel_decay: a_log")
+    _need(dt_bias.dtype == torch.float32 and dt_bias.numel() == heads * dim and dt_bias.is_contiguous(),
+          "channel_decay: dt_bias")
+    fn = _fn("recurrent", "vk_channel_decay", [_p, _ll, _p, _p, _i, _i, _i, _p, _ll, _p])
+    _status(fn(_ptr(raw), raw.stride(0), _ptr(a_log), _ptr(dt_bias), heads, dim, tokens, _ptr(out), out.stride(0),
+               _stream()), "channel_decay")
+
+
+def delta_rule(qkv: torch.Tensor, beta: torch.Tensor, decay: Optional[torch.Tensor], state: torch.Tensor,
                entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, kv_heads: int, dim: int,
-               heads: int, vdim: int, out: torch.Tensor, num_entries: int, short_entries: bool = False) -> None:
+               heads: int, vdim: int, out: torch.Tensor, num_entries: int, short_entries: bool = False,
+               channel_decay_col: int = -1) -> None:
     """The gated delta rule over every entry's tokens in order (``short_entries``: a step of single tokens, which
     takes the kernel's form with few registers; the result is the same), from and into the entries' state rows (the first
-    ``heads * recurrent_head_floats(dim, vdim)`` floats of a row, in the kernel's own order); ``out`` 32-bit ``[tokens, heads * vdim]``."""
+    ``heads * recurrent_head_floats(dim, vdim)`` floats of a row, in the kernel's own order); ``out`` 32-bit ``[tokens, heads * vdim]``.
+    ``decay`` is ``[tokens, heads]``; with ``channel_decay_col`` at or above 0 there is one decay per head and key
+    channel instead, ``[heads, dim]`` in every row of ``qkv`` from that column on (``qkv`` is then a view of the first
+    columns of those wider rows, and ``decay`` is None)."""
     _dev(qkv, beta, decay, state, entry_start, entry_first, slots, out)
     tokens = qkv.shape[0]
     channels = 2 * kv_heads * dim + heads * vdim
-    _need(qkv.shape == (tokens, channels) and beta.shape == (tokens, heads) and decay.shape == (tokens, heads)
-          and out.shape == (tokens, heads * vdim), "delta_rule: shapes")
-    for t in (qkv, beta, decay, out):
+    _need(qkv.shape == (tokens, channels) and qkv.dtype == torch.float32 and qkv.stride(1) == 1
+          and beta.shape == (tokens, heads) and out.shape == (tokens, heads * vdim), "delta_rule: shapes")
+    for t in (beta, out):
         _f32(t, "delta_rule: operands")
+    if channel_decay_col >= 0:
+        _need(decay is None and channel_decay_col >= channels and channel_decay_col + heads * dim <= qkv.stride(0),
+              "delta_rule: the decays per channel lie behind q, k and v inside the rows of qkv")
+    else:
+        _need(decay is not None and decay.shape == (tokens, heads) and qkv.stride(0) == channels, "delta_rule: decay")
+        _f32(decay, "delta_rule: decay")
     _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
           and state.shape[1] >= heads * recurrent_head_floats(dim, vdim), "delta_rule: state row")
     _entries_ok((entry_start, entry_first, slots), num_entries)
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"delta_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
-    fn = _fn("recurrent", "vk_delta_rule", [_p, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p])
-    _status(fn(_ptr(qkv), _ptr(beta), _ptr(decay), _ptr(state), state.stride(0), _ptr(entry_start), _ptr(entry_first),
-               _ptr(slots), kv_heads, dim, heads, vdim, _ptr(out), num_entries, 1 if short_entries else 0, _stream()),
-            "delta_rule")
+    fn = _fn("recurrent", "vk_delta_rule_strided", [_p, _ll, _i, _p, _p, _p, _ll, _p, _p, _p, _i, _i, _i, _i, _p, _i, _i, _p])
+    _status(fn(_ptr(qkv), qkv.stride(0), int(channel_decay_col), _ptr(beta), _ptr(decay), _ptr(state), state.stride(0),
+               _ptr(entry_start), _ptr(entry_first), _ptr(slots), kv_heads, dim, heads, vdim, _ptr(out), num_entries,
+               1 if short_entries else 0, _stream()), "delta_rule")
+
+
+def memory_state_floats(heads: int, dim: int, vdim: int) -> int:
+    """Floats of one request's matrix-memory state (:func:`memory_rule`): the heads' matrices, then the normalizer
+    vector and the running maximum once per tile of eight value channels."""
+    rows = 1 if dim <= 16 else 2 if dim <= 32 else 4 if dim <= 64 else 8 if dim <= 128 else 16
+    tiles = (vdim + 15) // 16 * 2
+    return heads * (recurrent_head_floats(dim, vdim) + tiles * 16 * rows + tiles)
+
+
+def memory_rule(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col: int, f_col: int, q_scale: float, cap: float,
+                state: torch.Tensor, entry_start: torch.Tensor, entry_first: torch.Tensor, slots: torch.Tensor, dim: int,
+                heads: int, vdim: int, out: torch.Tensor, num_entries: int, short_entries: bool = False) -> None:
+    """The matrix memory with exponential gates over every entry's tokens in order: with ``li = cap tanh(i / cap)``,
+    ``lf = logsigmoid(cap tanh(f / cap))`` and a running maximum ``m`` (0 at position 0): ``m' = max(lf + m, li)``,
+    ``S = exp(lf + m - m') S + exp(li - m') k v^T``, ``n`` likewise with ``k`` alone,
+    ``o = S^T q / (max(|n . q|, exp(-m')) + 1e-6)``.  q, k (``heads * dim`` each), v (``heads * vdim``) and the raw gates
+    (``heads`` each) are columns of the 32-bit ``proj`` from the given offsets on; q is multiplied by ``q_scale``.  State
+    rows hold :func:`memory_state_floats` floats; ``out`` 32-bit ``[tokens, heads * vdim]``."""
+    _dev(proj, state, entry_start, entry_first, slots, out)
+    tokens = proj.shape[0]
+    _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "memory_rule: proj")
+    _need(min(q_col, k_col, v_col, i_col, f_col) >= 0
+          and max(q_col + heads * dim, k_col + heads * dim, v_col + heads * vdim, i_col + heads, f_col + heads) <= proj.shape[1],
+          "memory_rule: columns")
+    _need(out.shape == (tokens, heads * vdim), "memory_rule: out shape")
+    _f32(out, "memory_rule: out")
+    _need(state.dim() == 2 and state.dtype == torch.float32 and state.is_contiguous()
+          and state.shape[1] >= memory_state_floats(heads, dim, vdim), "memory_rule: state row")
+    _entries_ok((entry_start, entry_first, slots), num_entries)
+    _need(cap > 0.0, "memory_rule: the gates' cap must be above 0")
+    if dim > RECURRENT_MAX_KEY_DIM:
+        raise UnsupportedError(f"memory_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
+    fn = _fn("recurrent", "vk_memory_rule", [_p, _ll, _i, _i, _i, _i, _i, _f, _f, _p, _ll, _p, _p, _p, _i, _i, _i, _p, _i, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), q_col, k_col, v_col, i_col, f_col, float(q_scale), float(cap), _ptr(state),
+               state.stride(0), _ptr(entry_start), _ptr(entry_first), _ptr(slots), dim, heads, vdim, _ptr(out),
+               num_entries, 1 if short_entries else 0, _stream()), "memory_rule")
 
 
 def wkv_rule(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, wraw: torch.Tensor, w0: torch.Tensor,
@@ -1065,17 +1134,18 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, ga
                    vdim: int, out: torch.Tensor) -> None:
     """``out[t, h] = o[t, h] / rms(o[t, h]) * weight * gate[t, h]`` per head of ``vdim`` channels; ``weight`` is
     ``[vdim]`` (shared by the heads) or ``[heads * vdim]``; ``gate`` (a row-strided view of either dtype) goes through
-    silu first if ``gate_silu``."""
+    silu first if ``gate_silu`` is true, or through the sigmoid if it is the string ``"sigmoid"``."""
     _dev(o, weight, gate, out)
     tokens = o.shape[0]
     _f32(o, "head_norm_gate: o")
+    gate_kind = 2 if gate_silu == "sigmoid" else 1 if gate_silu in (True, "silu") else 0
     _need(o.shape == (tokens, heads * vdim) and out.shape == o.shape and out.is_contiguous(), "head_norm_gate: shapes")
     _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() in (vdim, heads * vdim),
           "head_norm_gate: weight")
     _need(gate.shape == o.shape and gate.stride(1) == 1, "head_norm_gate: gate")
     fn = _fn("recurrent", "vk_head_norm_gate", [_p, _p, _i, _p, _i, _ll, _i, _f, _i, _i, _i, _p, _i, _p])
     _status(fn(_ptr(o), _ptr(weight), 1 if weight.numel() == heads * vdim and heads > 1 else 0, _ptr(gate),
-               _dt(gate, "gate"), gate.stride(0), 1 if gate_silu else 0, float(eps), heads, vdim, tokens, _ptr(out),
+               _dt(gate, "gate"), gate.stride(0), gate_kind, float(eps), heads, vdim, tokens, _ptr(out),
                _dt(out, "out"), _stream()), "head_norm_gate")
 
 
@@ -1145,12 +1215,13 @@ def moe_max_tiles(pairs: int, experts: int, tile_rows: int = 64) -> int:
 
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, offsets: torch.Tensor,
               order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, tile_rows: int = 64,
-              groups: int = 1, keep: int = 1, all_scores: bool = False) -> None:
+              groups: int = 1, keep: int = 1, all_scores=False) -> None:
     """Each token's ``top`` largest router logits (lowest id first among equals) with the softmax over those, and the
     (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``.
     ``groups`` > 1: the experts form that many equal groups of neighbours and only those of the ``keep`` groups with
     the largest logits can be chosen.  ``all_scores``: the weights are the chosen experts' shares of the softmax over
-    all experts (they do not add up to one)."""
+    all experts (they do not add up to one); ``all_scores="sigmoid"``: the weight of a chosen expert is the sigmoid of its
+    own logit, not renormalized."""
     _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
     tokens, experts = logits.shape
     _f32(logits, "moe_route: logits")
@@ -1163,17 +1234,18 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
     _need(1 <= keep <= groups <= 64 and experts % groups == 0 and (keep == groups or keep * (experts // groups) >= top),
           f"moe_route: {keep} of {groups} groups of {experts} experts for top {top}")
     fn = _fn("moe", "vk_moe_route_grouped", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
-    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), 1 if all_scores else 0, _ptr(ids),
+    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), 2 if all_scores == "sigmoid" else 1 if all_scores else 0, _ptr(ids),
                _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles), _ptr(num_tiles), _stream()), "moe_route")
 
 
 def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
                 order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, weights: torch.Tensor, top: int,
                 limit: float, alpha: float, act: torch.Tensor, pair_out: torch.Tensor, residual: torch.Tensor,
-                accumulate: bool = True) -> None:
+                accumulate: bool = True, weigh_input: bool = False) -> None:
     """The chosen experts of every token: ``y = g * sigmoid(alpha * g) * (u + 1)`` with ``g = min(Wg h, limit)`` and
     ``u = clamp(Wu h, -limit, limit)``, or with an infinite ``limit`` ``y = g * sigmoid(alpha * g) * u`` (alpha 1:
-    ``silu(g) * u``); then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])`` (without ``accumulate``: ``=``)."""
+    ``silu(g) * u``); then ``Wd y``; ``residual += sum_j weights[t, j] * expert_j(h[t])`` (without ``accumulate``: ``=``).
+    ``weigh_input``: ``residual += sum_j expert_j(weights[t, j] * h[t])`` instead."""
     _dev(h, w_gate, w_up, w_down, offsets, order, tiles, num_tiles, weights, act, pair_out, residual)
     tokens, width = h.shape
     experts, ff, _ = w_gate.shape
@@ -1191,11 +1263,12 @@ def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_dow
     _need(offsets.numel() == experts + 1 and order.numel() == tokens * top
           and tiles.numel() >= 2 * moe_max_tiles(tokens * top, experts, moe_tile_rows(h, width, ff)),
           "moe_experts: grouping (made by moe_route with moe_tile_rows(h, width, ff))")
-    fn = _fn("moe", "vk_moe_experts_into", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p, _p,
-                                            _i, _p])
+    fn = _fn("moe", "vk_moe_experts_weighed", [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _f, _p, _p,
+                                               _p, _i, _i, _p])
     _status(fn(_ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _dt(h, "h"), _ptr(offsets), _ptr(order),
                _ptr(tiles), _ptr(num_tiles), _ptr(weights), tokens, experts, top, width, ff, float(limit), float(alpha),
-               _ptr(act), _ptr(pair_out), _ptr(residual), 1 if accumulate else 0, _stream()), "moe_experts")
+               _ptr(act), _ptr(pair_out), _ptr(residual), 1 if accumulate else 0, 1 if weigh_input else 0, _stream()),
+            "moe_experts")
 
 
 # --- norms behind a sublayer, sums of two streams, activations ------------------------------------------
@@ -1274,6 +1347,35 @@ def whole_norm_pack(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weig
     fn = _fn("elementwise", "vk_whole_norm_pack", [_p, _ll, _p, _p, _f, _i, _i, _i, _i, _i, _i, _p, _i, _p])
     _status(fn(_ptr(proj), proj.stride(0), _ptr(q_weight), _ptr(k_weight), float(eps), tokens, heads, kv_heads, dim, vdim,
                padded, _ptr(qkv), _dt(qkv, "qkv"), _stream()), "whole_norm_pack")
+
+
+def head_norm_pack(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], eps: float,
+                   heads: int, kv_heads: int, dim: int, vdim: int, padded: int, qkv: torch.Tensor,
+                   first: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None) -> None:
+    """From the 32-bit sums ``proj [T, >= q | k | v]``: every q head and every k head divided by its own root mean square
+    and multiplied by a weight of ``dim`` numbers that the heads share (None: left as they are); with ``first`` (32-bit
+    ``[T, kv_heads * vdim]``, row-strided) the values become ``(1 - mix) v + mix first``, ``mix`` one number on the
+    device; q, k and v laid out head by head, each padded with zeros to ``padded`` columns."""
+    _dev(proj, q_weight, k_weight, qkv, first, mix)
+    _f32s(proj, "head_norm_pack: proj")
+    tokens = qkv.shape[0]
+    need = (heads + kv_heads) * dim + kv_heads * vdim
+    _need(proj.dim() == 2 and proj.shape[0] == tokens and proj.shape[1] >= need and proj.stride(1) == 1,
+          "head_norm_pack: proj")
+    _need(padded >= max(dim, vdim) and qkv.shape == (tokens, (heads + 2 * kv_heads) * padded) and qkv.is_contiguous(),
+          "head_norm_pack: qkv")
+    for weight in (q_weight, k_weight):
+        if weight is not None:
+            _need(weight.dtype == torch.float32 and weight.numel() == dim and weight.is_contiguous(),
+                  "head_norm_pack: a weight per number of a head")
+    if first is not None:
+        _need(first.dtype == torch.float32 and first.shape == (tokens, kv_heads * vdim) and first.stride(1) == 1,
+              "head_norm_pack: first")
+        _need(mix is not None and mix.dtype == torch.float32 and mix.numel() == 1, "head_norm_pack: mix must be one float32")
+    fn = _fn("elementwise", "vk_head_norm_pack", [_p, _ll, _p, _p, _f, _p, _ll, _p, _i, _i, _i, _i, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(first),
+               first.stride(0) if first is not None else 0, _ptr(mix) if first is not None else None, tokens, heads,
+               kv_heads, dim, vdim, padded, _ptr(qkv), _dt(qkv, "qkv"), _stream()), "head_norm_pack")
 
 
 def head_unpack_gate(attn: torch.Tensor, gate: Optional[torch.Tensor], gate_kind: str, heads: int, vdim: int,

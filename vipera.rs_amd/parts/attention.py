@@ -9,11 +9,16 @@ the concatenated weight ``[Wq; Wk; Wv]``, whose rows equal the separate products
 Options, each a parameter that any architecture may set: ``softcap`` (a score becomes ``softcap * tanh(score /
 softcap)``); ``chunk`` (a token sees the earlier tokens of its own block of that many positions, blocks counted from
 position 0, instead of a window); ``value_dim`` (values narrower or wider than keys); ``qk_norm: "whole"`` (q and k
-each RMS-normed over the whole projection, all heads at once, with a weight per number, before the rotation);
-``gate: "sigmoid"`` (the heads' outputs times ``sigmoid(Wg h)`` before the output projection); ``tensors`` (the
-tensors' names after the part's name).  With any of the last three the step runs as one product ``[q | k | v | g]`` with
-32-bit sums, a kernel that norms and lays the heads out at one padded width, the rotation with the cache write, the
-paged attention kernels at that width, and a kernel that unpacks and gates.
+each RMS-normed over the whole projection, all heads at once, with a weight per number, before the rotation) or
+``qk_norm: "head"`` (every q head and every k head RMS-normed by itself, with one weight of ``head_dim`` numbers for
+all q heads and one for all k heads); ``gate: "sigmoid"`` (the heads' outputs times ``sigmoid(Wg h)`` before the output
+projection); ``value_mix`` (``"source"``: the layer's values of the step's tokens are kept for later layers;
+``"blend"``: its values become ``(1 - l) v + l v_source`` with the learned number ``l`` and the source layer's values
+of the same token, and the blended values are what is cached; a ``"source"`` layer declares the number too and does not
+read it); ``tensors`` (the tensors' names after the part's name).  With any of these but the first three the step runs
+as one product ``[q | k | v | g]`` with 32-bit sums (biases added there), a kernel that norms and lays the heads out at
+one padded width, the rotation with the cache write, the paged attention kernels at that width, and a kernel that
+unpacks and gates.
 """
 from __future__ import annotations
 
@@ -39,7 +44,11 @@ def _cat(tensors: List[torch.Tensor]) -> torch.Tensor:
 
 
 _DEFAULT_NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
-                  "g": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight"}
+                  "g": "g_proj.weight", "q_norm": "q_norm.weight", "k_norm": "k_norm.weight",
+                  "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias",
+                  "value_mix": "value_mix"}
+
+VALUE_MIX_KEY = "attention.value_mix.source"    # where a step keeps the source layer's values (``batch.shared``)
 
 
 def _tensor_names(p) -> Dict[str, str]:
@@ -50,7 +59,8 @@ def _tensor_names(p) -> Dict[str, str]:
 
 def _is_general(p) -> bool:
     """Whether the layer needs the path that norms, pads and gates (see the module's text)."""
-    return bool(p.get("qk_norm") or p.get("gate") or int(p.get("value_dim") or p["head_dim"]) != int(p["head_dim"]))
+    return bool(p.get("qk_norm") or p.get("gate") or p.get("value_mix")
+                or int(p.get("value_dim") or p["head_dim"]) != int(p["head_dim"]))
 
 
 def _padded_width(p) -> int:
@@ -79,18 +89,18 @@ class Attention(Mixer):
             raise InvalidArgumentError("attention: a window and blocks of positions exclude each other")
         self.mask = -self.chunk if self.chunk else self.window      # what the kernels take as `window`
         self.value_dim = int(p.get("value_dim") or self.head_dim)
-        self.qk_norm, self.gate = p.get("qk_norm"), p.get("gate")
+        self.qk_norm, self.gate, self.value_mix = p.get("qk_norm"), p.get("gate"), p.get("value_mix")
         self.general = _is_general(p)
         self.padded = _padded_width(p)
-        if self.general and (self.qkv_bias or self.out_bias):
-            raise UnsupportedError("attention: biases with value_dim, qk_norm or gate are not implemented")
+        if self.gate and self.qkv_bias:
+            raise UnsupportedError("attention: biases on q, k and v beside an output gate are not implemented")
         scale = p.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
         if self.heads % self.kv_heads:
             raise InvalidArgumentError(f"heads {self.heads} is not a multiple of kv_heads {self.kv_heads}")
         self.q_width = self.heads * self.head_dim
         self.kv_width = self.kv_heads * self.head_dim
-        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = self.q_norm = self.k_norm = self.mix = None
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
@@ -104,13 +114,16 @@ class Attention(Mixer):
         for name, rows in (("q", q), ("k", kv), ("v", int(p["kv_heads"]) * vd)):
             specs.append(TensorSpec(base + names[name], (rows, hidden), MATRIX))
             if p.get("qkv_bias"):
-                specs.append(TensorSpec(f"{base}{name}_proj.bias", (rows,), VECTOR))
+                specs.append(TensorSpec(base + names[name + "_bias"], (rows,), VECTOR))
         specs.append(TensorSpec(base + names["o"], (hidden, int(p["heads"]) * vd), MATRIX))
         if p.get("out_bias"):
-            specs.append(TensorSpec(base + "o_proj.bias", (hidden,), VECTOR))
+            specs.append(TensorSpec(base + names["o_bias"], (hidden,), VECTOR))
         if p.get("qk_norm"):
-            specs += [TensorSpec(base + names["q_norm"], (q,), VECTOR, "one_plus_normal"),
-                      TensorSpec(base + names["k_norm"], (kv,), VECTOR, "one_plus_normal")]
+            per_head = p.get("qk_norm") == "head"
+            specs += [TensorSpec(base + names["q_norm"], (hd if per_head else q,), VECTOR, "one_plus_normal"),
+                      TensorSpec(base + names["k_norm"], (hd if per_head else kv,), VECTOR, "one_plus_normal")]
+        if p.get("value_mix"):
+            specs.append(TensorSpec(base + names["value_mix"], (), VECTOR, std=0.3))
         if p.get("gate"):
             specs.append(TensorSpec(base + names["g"], (int(p["heads"]) * vd, hidden), MATRIX))
         return specs
@@ -123,12 +136,14 @@ class Attention(Mixer):
             parts.append(tensors[base + names["g"]])
         self.w_qkv = _cat(parts)
         if self.qkv_bias:
-            self.b_qkv = torch.cat([tensors[base + f"{n}_proj.bias"] for n in "qkv"]).contiguous()
+            self.b_qkv = torch.cat([tensors[base + names[n + "_bias"]] for n in "qkv"]).contiguous()
         self.w_o = tensors[base + names["o"]]
         if self.out_bias:
-            self.b_o = tensors[base + "o_proj.bias"]
+            self.b_o = tensors[base + names["o_bias"]]
         if self.qk_norm:
             self.q_norm, self.k_norm = tensors[base + names["q_norm"]], tensors[base + names["k_norm"]]
+        if self.value_mix:
+            self.mix = tensors[base + names["value_mix"]].reshape(1)
 
     @classmethod
     def declare_cache(cls, spec: PartSpec):
@@ -141,8 +156,11 @@ class Attention(Mixer):
     def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
         p = spec.params
         heads, kv_heads, head_dim = int(p["heads"]), int(p["kv_heads"]), _padded_width(p)
-        if p.get("qk_norm") not in (None, "whole"):
-            raise UnsupportedError(f"attention: qk_norm {p.get('qk_norm')!r} is not implemented; \"whole\" or none")
+        if p.get("qk_norm") not in (None, "whole", "head"):
+            raise UnsupportedError(f"attention: qk_norm {p.get('qk_norm')!r} is not implemented; \"whole\", \"head\" or none")
+        if p.get("value_mix") not in (None, "source", "blend"):
+            raise UnsupportedError(f"attention: value_mix {p.get('value_mix')!r} is not implemented; \"source\", "
+                                   "\"blend\" or none")
         if p.get("gate") not in (None, "sigmoid", "silu"):
             raise UnsupportedError(f"attention: gate {p.get('gate')!r} is not implemented; \"sigmoid\", \"silu\" or none")
         if head_dim > kernels.ATTENTION_MAX_HEAD_DIM:
@@ -184,10 +202,29 @@ class Attention(Mixer):
         tokens = residual.shape[0]
         width = self.padded
         proj = torch.empty((tokens, self.w_qkv.shape[0]), dtype=torch.float32, device=residual.device)
-        linear(h, self.w_qkv, None, proj)
+        linear(h, self.w_qkv, self.b_qkv, proj)
         qkv = self.runtime.empty((tokens, (self.heads + 2 * self.kv_heads) * width))
-        kernels.whole_norm_pack(proj, self.q_norm, self.k_norm, float(self.spec.params.get("eps") or 0.0), self.heads,
-                                self.kv_heads, self.head_dim, self.value_dim, width, qkv)
+        eps = float(self.spec.params.get("eps") or 0.0)
+        first = None
+        if self.value_mix:
+            # the source layer's values of the step's tokens, as its product left them, are kept for the step
+            v_col = (self.heads + self.kv_heads) * self.head_dim
+            mine = proj[:, v_col:v_col + self.kv_heads * self.value_dim]
+            if self.value_mix == "source":
+                batch.shared[VALUE_MIX_KEY] = mine
+            else:
+                first = batch.shared.get(VALUE_MIX_KEY)
+                if first is None or first.shape != mine.shape:
+                    raise InvalidArgumentError("attention: a layer blends its values with a source layer's, but no layer "
+                                               "before it in the run order keeps values of this shape")
+        if self.qk_norm == "whole" and first is None:
+            kernels.whole_norm_pack(proj, self.q_norm, self.k_norm, eps, self.heads, self.kv_heads, self.head_dim,
+                                    self.value_dim, width, qkv)
+        elif self.qk_norm == "whole":
+            raise UnsupportedError("attention: value_mix beside qk_norm \"whole\" is not implemented")
+        else:
+            kernels.head_norm_pack(proj, self.q_norm, self.k_norm, eps, self.heads, self.kv_heads, self.head_dim,
+                                   self.value_dim, width, qkv, first, self.mix if first is not None else None)
         table = batch.block_tables[cache.group]
         fused = position.fused_rotary()
         inv_freq, rotary_dim = fused if fused is not None else (None, 0)
@@ -206,7 +243,7 @@ class Attention(Mixer):
         values = self.runtime.empty((tokens, self.heads * self.value_dim))
         gate = proj[:, (self.heads + self.kv_heads) * self.head_dim + self.kv_heads * self.value_dim:] if self.gate else None
         kernels.head_unpack_gate(attn, gate, self.gate or "none", self.heads, self.value_dim, width, values)
-        linear(values, self.w_o, None, residual, accumulate=accumulate)
+        linear(values, self.w_o, self.b_o, residual, accumulate=accumulate)
 
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, handoff=None,
                 incoming=None, accumulate: bool = True) -> None:

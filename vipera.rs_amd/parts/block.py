@@ -2,7 +2,8 @@
 
 ``prenorm``: ``x += mixer(norm_1(x)); x += ffn(norm_2(x))``, the pre-norm residual block of the
 reference (crates/vipera-backend-cpu/src/model.rs:3-4, 975-1198).
-``parallel``: ``h = norm(x); x += mixer(h) + ffn(h)``.
+``parallel``: ``h = norm(x); x += mixer(h) + ffn(h)``; with a second norm of its own for the feed-forward,
+``x += m * (mixer(norm_1(x)) + ffn(norm_2(x)))``, both norms of the same ``x``, ``m`` = ``params["residual_mult"]``.
 ``sandwich_norm``: a norm before and behind each sublayer, ``x += norm_1b(mixer(norm_1(x))); x += norm_2b(ffn(norm_2(x)))``,
 and optionally a part that adds to the stream after both (``extras["after"]``, of the feed-forward family; it reads the
 32-bit stream itself).  The norms behind the sublayers are ``extras["mixer_post_norm"]`` and ``extras["ffn_post_norm"]``.
@@ -77,7 +78,9 @@ class PreNormBlock(Block):
 
 class ParallelBlock(Block):
     """``h = norm(x); x += mixer(h) + ffn(h)``: one norm, and both sublayers read its output.  The layer's norm is
-    ``LayerSpec.mixer_norm``; ``ffn_norm`` is not read."""
+    ``LayerSpec.mixer_norm``.  Where ``ffn_norm`` is another norm than ``mixer_norm`` (another tensor name) the
+    feed-forward reads that one, of the same ``x``.  ``LayerSpec.params["residual_mult"]`` (1 unless given) multiplies the
+    sublayers' sum: they then add into a 32-bit buffer of their own, which joins the stream in one step."""
 
     def __init__(self, spec: LayerSpec, runtime):
         super().__init__(spec, runtime)
@@ -85,16 +88,33 @@ class ParallelBlock(Block):
         self.mixer = part_class("mixer", spec.mixer.kind)(spec.mixer, spec.prefix, runtime)
         self.ffn = part_class("ffn", spec.ffn.kind)(spec.ffn, spec.prefix, runtime)
         self.position = part_class("position", spec.position.kind)(spec.position, spec.prefix, runtime)
+        self.has_ffn = spec.ffn.kind != "none"
+        self.ffn_norm = None
+        if self._two_norms(spec):
+            self.ffn_norm = part_class("norm", spec.ffn_norm.kind)(spec.ffn_norm, spec.prefix, runtime)
+        self.mult = float(spec.params.get("residual_mult", 1.0))
+
+    @staticmethod
+    def _two_norms(spec: LayerSpec) -> bool:
+        return spec.ffn.kind != "none" and spec.ffn_norm != spec.mixer_norm
 
     @classmethod
     def _families(cls, spec: LayerSpec):
-        return (("norm", spec.mixer_norm), ("mixer", spec.mixer), ("ffn", spec.ffn), ("position", spec.position))
+        parts = [("norm", spec.mixer_norm), ("mixer", spec.mixer), ("ffn", spec.ffn), ("position", spec.position)]
+        if cls._two_norms(spec):
+            parts.append(("norm", spec.ffn_norm))
+        return parts
 
     @classmethod
     def declare(cls, spec: LayerSpec) -> List[TensorSpec]:
         out: List[TensorSpec] = []
         for family, part in cls._families(spec):
             out += part_class(family, part.kind).declare(part, spec.prefix)
+        if spec.ffn.kind == "none" and spec.ffn_norm != spec.mixer_norm:
+            # a layer without a feed-forward does not read the norm in front of it; a folder that stores it all the
+            # same is not refused for it
+            out += [TensorSpec(t.name, t.shape, t.role, t.init, t.std, True)
+                    for t in part_class("norm", spec.ffn_norm.kind).declare(spec.ffn_norm, spec.prefix)]
         return out
 
     @classmethod
@@ -103,14 +123,28 @@ class ParallelBlock(Block):
             part_class(family, part.kind).check_supported(part, dtype)
 
     def load(self, tensors) -> None:
-        for part in (self.norm, self.mixer, self.ffn, self.position):
-            part.load(tensors)
+        for part in (self.norm, self.mixer, self.ffn, self.position, self.ffn_norm):
+            if part is not None:
+                part.load(tensors)
 
     def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
-        # both sublayers add into the 32-bit residual; neither reads it, so their order does not matter
         h = self.norm.forward(x)
-        self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
-        self.ffn.forward(h, batch, x)
+        h_ffn = self.ffn_norm.forward(x) if self.ffn_norm is not None else h
+        if self.mult == 1.0:
+            # both sublayers add into the 32-bit residual; neither reads it after the norms, so their order does not matter
+            self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
+            self.ffn.forward(h_ffn, batch, x)
+            return
+        import torch
+        from ..ops import kernels
+        if self.mixer.can_overwrite:
+            y = torch.empty_like(x)
+            self.mixer.forward(h, batch, cache, state, self.position, y, reads_only, accumulate=False)
+        else:
+            y = torch.zeros_like(x)
+            self.mixer.forward(h, batch, cache, state, self.position, y, reads_only)
+        self.ffn.forward(h_ffn, batch, y)
+        kernels.axpby(y, self.mult, y, 0.0, x, accumulate=True)      # x += m * y
 
 
 class SandwichBlock(Block):

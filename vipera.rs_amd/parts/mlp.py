@@ -20,6 +20,16 @@ from .base import FeedForward, register_ffn
 
 
 class GatedMLP(FeedForward):
+    """``params``: ``hidden``, ``intermediate``, ``name``; tensors ``<name>.gate_proj.weight | up_proj.weight |
+    down_proj.weight``, or as ``params["tensors"]`` names them (keys ``gate``, ``up``, ``down``)."""
+
+    @staticmethod
+    def _names(spec: PartSpec, prefix: str):
+        names = {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        names.update(spec.params.get("tensors") or {})
+        base = f"{prefix}{spec.params['name']}."
+        return base + names["gate"], base + names["up"], base + names["down"]
+
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
         self.hidden = int(spec.params["hidden"])
@@ -31,22 +41,22 @@ class GatedMLP(FeedForward):
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
-        base = f"{prefix}{spec.params['name']}."
+        gate, up, down = cls._names(spec, prefix)
         hidden, inter = int(spec.params["hidden"]), int(spec.params["intermediate"])
         return [
-            TensorSpec(base + "gate_proj.weight", (inter, hidden), MATRIX),
-            TensorSpec(base + "up_proj.weight", (inter, hidden), MATRIX),
-            TensorSpec(base + "down_proj.weight", (hidden, inter), MATRIX),
+            TensorSpec(gate, (inter, hidden), MATRIX),
+            TensorSpec(up, (inter, hidden), MATRIX),
+            TensorSpec(down, (hidden, inter), MATRIX),
         ]
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
-        base = f"{self.prefix}{self.spec.params['name']}."
-        gate, up = tensors[base + "gate_proj.weight"], tensors[base + "up_proj.weight"]
+        gate_name, up_name, down_name = self._names(self.spec, self.prefix)
+        gate, up = tensors[gate_name], tensors[up_name]
         # all-bfloat16 weights of a width the kernels can pair are interleaved, so that the product's
         # epilogue can apply the gate; anything else stays [gate; up]
         self.interleaved = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0)
         self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
-        self.w_down = tensors[base + "down_proj.weight"]
+        self.w_down = tensors[down_name]
 
     def _dividing_plan(self, tokens: int):
         """0 or 3 where the gate/up product of ``tokens`` rows runs on a kernel that can divide by the norm in front

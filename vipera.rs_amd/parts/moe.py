@@ -7,7 +7,10 @@ adds the weighted sum of the chosen experts' outputs to the residual.  ``limit``
 a ``limit`` nothing is clamped and ``y = g * sigmoid(alpha * g) * u`` (``alpha`` 1: ``silu(g) * u``).  ``groups`` and
 ``keep``: the experts form that many equal groups of neighbours, a group's score is its largest logit, and only experts
 of the ``keep`` best groups can be chosen.  ``scores: "all"``: the weights are the chosen experts' shares of the softmax
-over all experts, not renormalized.
+over all experts, not renormalized; ``scores: "sigmoid"``: a chosen expert's weight is the sigmoid of its own logit, not
+renormalized.  ``weigh: "input"``: the weight multiplies what the expert reads instead of what it returns, so the layer
+adds the sum of ``expert(w h)``.  ``shared``: a gated feed-forward of that width (``silu(Wg h) * (Wu h)`` through
+``Wd``, tensors ``<name>.shared.gate | up | down``) that every token runs beside its experts.
 
 The step's (token, choice) pairs are grouped by expert on the device, so nothing about the routing reaches the
 host and a step of single tokens can be captured; see ``csrc/kernels/moe.hip``.
@@ -28,8 +31,9 @@ from .base import FeedForward, register_ffn
 
 class MixtureOfExperts(FeedForward):
     """``params``: ``hidden``, ``intermediate`` (an expert's width), ``experts``, ``top``, ``limit`` (None: no clamp),
-    ``alpha`` (1.702 unless given), ``groups`` and ``keep`` (1 and 1 unless given), ``scores`` ("chosen" or "all"),
-    ``name``; tensors ``<name>.router`` and ``<name>.e<i>.gate | up | down``."""
+    ``alpha`` (1.702 unless given), ``groups`` and ``keep`` (1 and 1 unless given), ``scores`` ("chosen", "all" or
+    "sigmoid"), ``weigh`` ("output" or "input"), ``shared`` (the shared expert's width, or None), ``name``; tensors
+    ``<name>.router``, ``<name>.e<i>.gate | up | down`` and ``<name>.shared.gate | up | down``."""
 
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
@@ -39,10 +43,21 @@ class MixtureOfExperts(FeedForward):
         self.limit = float(p["limit"]) if p.get("limit") is not None else float("inf")
         self.alpha = float(p.get("alpha", 1.702))
         self.groups, self.keep = int(p.get("groups") or 1), int(p.get("keep") or p.get("groups") or 1)
-        self.all_scores = p.get("scores", "chosen") == "all"
+        self.all_scores = {"chosen": False, "all": True, "sigmoid": "sigmoid"}[p.get("scores", "chosen")]
+        self.weigh_input = p.get("weigh", "output") == "input"
+        self.shared = None
+        if p.get("shared"):
+            from .mlp import GatedMLP
+            self.shared = GatedMLP(self._shared_spec(p), prefix, runtime)
         if not 1 <= self.top <= self.experts:
             raise InvalidArgumentError(f"a token cannot use {self.top} of {self.experts} experts")
         self.w_router = self.w_gate = self.w_up = self.w_down = None
+
+    @staticmethod
+    def _shared_spec(p) -> PartSpec:
+        return PartSpec("gated_mlp", {"hidden": int(p["hidden"]), "intermediate": int(p["shared"]),
+                                      "name": f"{p['name']}.shared",
+                                      "tensors": {"gate": "gate", "up": "up", "down": "down"}})
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
@@ -55,6 +70,9 @@ class MixtureOfExperts(FeedForward):
                       TensorSpec(f"{base}e{e}.up", (inter, hidden), MATRIX),
                       TensorSpec(f"{base}e{e}.down", (hidden, inter), MATRIX)]
         specs.append(TensorSpec(base + "router", (int(p["experts"]), hidden), MATRIX))
+        if p.get("shared"):
+            from .mlp import GatedMLP
+            specs += GatedMLP.declare(cls._shared_spec(p), prefix)
         return specs
 
     @classmethod
@@ -70,8 +88,11 @@ class MixtureOfExperts(FeedForward):
         if groups < 1 or experts % groups or not 1 <= keep <= groups or (keep < groups and keep * (experts // groups) < top):
             raise InvalidArgumentError(f"mixture of experts: {keep} of {groups} groups of {experts} experts cannot "
                                        f"give a token its {top}")
-        if spec.params.get("scores", "chosen") not in ("chosen", "all"):
-            raise UnsupportedError(f"mixture of experts: scores {spec.params.get('scores')!r}; \"chosen\" or \"all\"")
+        if spec.params.get("scores", "chosen") not in ("chosen", "all", "sigmoid"):
+            raise UnsupportedError(f"mixture of experts: scores {spec.params.get('scores')!r}; \"chosen\", \"all\" or "
+                                   "\"sigmoid\"")
+        if spec.params.get("weigh", "output") not in ("output", "input"):
+            raise UnsupportedError(f"mixture of experts: weigh {spec.params.get('weigh')!r}; \"output\" or \"input\"")
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
@@ -79,6 +100,8 @@ class MixtureOfExperts(FeedForward):
         stack = lambda kind: torch.stack([tensors[f"{base}e{e}.{kind}"].to(dtype) for e in range(self.experts)]).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         self.w_router = tensors[base + "router"]
+        if self.shared is not None:
+            self.shared.load(tensors)
 
     can_overwrite = True
 
@@ -101,7 +124,9 @@ class MixtureOfExperts(FeedForward):
         act = self.runtime.empty((pairs, self.inter))
         pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
         kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,
-                            self.top, self.limit, self.alpha, act, pair_out, residual, accumulate)
+                            self.top, self.limit, self.alpha, act, pair_out, residual, accumulate, self.weigh_input)
+        if self.shared is not None:
+            self.shared.forward(h, batch, residual)
 
 
 register_ffn("moe", MixtureOfExperts)

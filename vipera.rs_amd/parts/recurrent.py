@@ -4,7 +4,18 @@
 (``heads x vdim``); each passes a short causal convolution over time per channel and silu; q and k become unit
 vectors per head (q also times ``dim^-1/2``); ``beta = sigmoid(Wb h)``, ``g = exp(-exp(A_log) softplus(Wa h +
 dt_bias))`` per head; then per head ``S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``; the read-out is
-``o / rms(o) * norm * silu(Wg h)`` and goes through ``Wo``.
+``o / rms(o) * norm * silu(Wg h)`` and goes through ``Wo``.  Options: ``decay: "channel"`` (one decay per head and key
+channel, ``g[h, d]``, which scales row ``d`` of ``S``; ``dt_bias`` is then ``[heads * dim]``), ``decay_rank`` and
+``gate_rank`` (the decay's and the gate's projections in two steps, ``Wa2 (Wa1 h)`` and ``Wg2 (Wg1 h)``, through that
+many numbers), ``gate: "sigmoid"``.
+
+``matrix_memory``: the matrix memory with exponential gates (mLSTM; Beck et al., "xLSTM: Extended Long Short-Term
+Memory").  ``q = Wq h * dim^-1/2``, ``k = Wk h`` (``heads x dim``), ``v = Wv h`` (``heads x vdim``); per head the
+logarithms of an input gate ``li = cap tanh((Wi h + bi) / cap)`` and of a forget gate
+``lf = logsigmoid(cap tanh((Wf h + bf) / cap))``; with a running maximum ``m`` that starts at 0:
+``m' = max(lf + m, li); S <- exp(lf + m - m') S + exp(li - m') k v^T``, ``n`` likewise with ``k`` alone,
+``o = S^T q / (max(|n . q|, exp(-m')) + 1e-6)``; the read-out is ``o / rms(o)`` per head ``* norm * sigmoid(Wg h)`` and
+goes through ``Wo``.
 
 ``wkv``: RWKV-style time mixing.  Each of r, k, v, g, w reads its own mix ``h + (h_prev - h) * mu``; the decay is
 ``w = exp(-exp(W2 tanh(W1 mix_w) + w0))`` per key channel; per head ``o = (S + diag(u) k v^T)^T r`` and then
@@ -43,7 +54,12 @@ UNIT_EPS = 1e-6   # q and k of the delta rule: x / sqrt(sum(x^2) + UNIT_EPS)
 
 class GatedDelta(Mixer):
     """``params``: ``hidden``, ``heads``, ``kv_heads``, ``dim``, ``vdim``, ``conv`` (taps), ``eps`` (of the read-out's
-    norm), ``name``."""
+    norm), ``name``; optional ``decay`` ("head": one per head, tensors ``a`` ``[heads, hidden]`` and ``dt_bias``
+    ``[heads]``; "channel": one per head and key channel, ``heads * dim`` of each), ``decay_rank`` and ``gate_rank``
+    (0: one projection ``a`` / ``g``; a number: two, ``a1`` ``[rank, hidden]`` and ``a2`` ``[., rank]``, ``g1`` and
+    ``g2``; -1: as many as the folder's tensor has), ``gate`` ("silu" or "sigmoid")."""
+
+    can_overwrite = True
 
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
@@ -55,7 +71,11 @@ class GatedDelta(Mixer):
             raise InvalidArgumentError(f"heads {self.heads} is not a multiple of kv_heads {self.kv_heads}")
         self.qk, self.vw = self.kv_heads * self.dim, self.heads * self.vdim
         self.channels = 2 * self.qk + self.vw
-        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = None
+        self.per_channel = p.get("decay", "head") == "channel"
+        self.decays = self.heads * self.dim if self.per_channel else self.heads
+        self.decay_rank, self.gate_rank = int(p.get("decay_rank") or 0), int(p.get("gate_rank") or 0)
+        self.gate_kind = p.get("gate", "silu")
+        self.w_in = self.w_o = self.conv = self.a_log = self.dt_bias = self.norm = self.w_a2 = self.w_g2 = None
 
     @classmethod
     def _sizes(cls, p):
@@ -68,14 +88,20 @@ class GatedDelta(Mixer):
         base = f"{prefix}{p['name']}."
         hidden, heads, taps = int(p["hidden"]), int(p["heads"]), int(p["conv"])
         qk, vw, _ = cls._sizes(p)
+        decays = heads * int(p["dim"]) if p.get("decay", "head") == "channel" else heads
         specs = []
         for name, rows in (("q", qk), ("k", qk), ("v", vw)):
             specs.append(TensorSpec(base + name, (rows, hidden), MATRIX))
             specs.append(TensorSpec(f"{base}{name}.conv", (rows, taps), VECTOR, std=0.5))
         specs += [TensorSpec(base + "b", (heads, hidden), MATRIX), TensorSpec(base + "A_log", (heads,), VECTOR),
                   TensorSpec(base + "norm", (int(p["vdim"]),), VECTOR, "one_plus_normal"),
-                  TensorSpec(base + "a", (heads, hidden), MATRIX), TensorSpec(base + "dt_bias", (heads,), VECTOR),
-                  TensorSpec(base + "g", (vw, hidden), MATRIX), TensorSpec(base + "o", (hidden, vw), MATRIX)]
+                  TensorSpec(base + "dt_bias", (decays,), VECTOR), TensorSpec(base + "o", (hidden, vw), MATRIX)]
+        for letter, rows, rank in (("a", decays, int(p.get("decay_rank") or 0)), ("g", vw, int(p.get("gate_rank") or 0))):
+            if rank:
+                specs += [TensorSpec(f"{base}{letter}1", (rank, hidden), MATRIX),
+                          TensorSpec(f"{base}{letter}2", (rows, rank), MATRIX, std=0.2)]
+            else:
+                specs.append(TensorSpec(base + letter, (rows, hidden), MATRIX))
         return specs
 
     @classmethod
@@ -95,36 +121,138 @@ class GatedDelta(Mixer):
             raise UnsupportedError(f"gated_delta: the convolution needs at least one tap, got {p['conv']}")
         if cls._sizes(p)[2] > 16_384:
             raise UnsupportedError("gated_delta: more than 16,384 convolved channels do not fit the kernel's LDS row")
+        if p.get("decay", "head") not in ("head", "channel") or p.get("gate", "silu") not in ("silu", "sigmoid"):
+            raise UnsupportedError(f"gated_delta: decay {p.get('decay')!r} with gate {p.get('gate')!r} is not implemented")
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
-        # one product for everything that reads h: [q | k | v | g | b | a] rows
-        self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", "g", "b", "a")])
+        # one product for everything that reads h: [q | k | v | g or g1 | b | a or a1] rows
+        gate, decay = ("g1" if self.gate_rank else "g"), ("a1" if self.decay_rank else "a")
+        self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", gate, "b", decay)])
+        self.gate_rows, self.decay_rows = int(tensors[base + gate].shape[0]), int(tensors[base + decay].shape[0])
+        if self.gate_rank:
+            self.w_g2 = tensors[base + "g2"]
+        if self.decay_rank:
+            self.w_a2 = tensors[base + "a2"]
+        for name, second, first_rows in (("g", self.w_g2, self.gate_rows), ("a", self.w_a2, self.decay_rows)):
+            if second is not None and second.shape[1] != first_rows:
+                raise InvalidArgumentError(f"{base}{name}2 has {second.shape[1]} columns for the {first_rows} rows of "
+                                           f"{base}{name}1")
         self.conv = torch.cat([tensors[f"{base}{n}.conv"] for n in ("q", "k", "v")]).contiguous()
         self.a_log, self.dt_bias, self.norm = tensors[base + "A_log"], tensors[base + "dt_bias"], tensors[base + "norm"]
         self.w_o = tensors[base + "o"]
 
-    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False) -> None:
+    def _second_step(self, low: torch.Tensor, weight: torch.Tensor, out_dtype) -> torch.Tensor:
+        """``weight`` applied to the 32-bit columns ``low`` of the first product: in the run's dtype, as every product."""
+        tokens = low.shape[0]
+        rows = self.runtime.empty((tokens, low.shape[1]))
+        kernels.activation(low, "none", rows)
+        out = torch.empty((tokens, weight.shape[0]), dtype=out_dtype, device=low.device)
+        linear(rows, weight, None, out)
+        return out
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
         tokens, entries = residual.shape[0], batch.num_entries
         device = residual.device
         f32 = dict(dtype=torch.float32, device=device)
         # what enters the recurrence stays 32-bit from the product's sums on
         proj = torch.empty((tokens, self.w_in.shape[0]), **f32)
         linear(h, self.w_in, None, proj)
-        qkv = torch.empty((tokens, self.channels), **f32)
-        beta, decay = torch.empty((tokens, self.heads), **f32), torch.empty((tokens, self.heads), **f32)
         g_col = self.channels
-        b_col = g_col + self.vw
+        b_col = g_col + self.gate_rows
+        a_col = b_col + self.heads
+        plain = not self.per_channel and not self.decay_rank       # the decay per head straight from the first product
+        # q, k, v and, behind them, the decays per key channel where the layer has those
+        rows = torch.empty((tokens, self.channels + (self.decays if self.per_channel else 0)), **f32)
+        qkv = rows[:, :self.channels]
+        beta = torch.empty((tokens, self.heads), **f32)
+        decay = None if self.per_channel else torch.empty((tokens, self.heads), **f32)
         matrices = self.heads * kernels.recurrent_head_floats(self.dim, self.vdim)
         kernels.delta_prepare(proj, self.conv, state, matrices, batch.entry_of_token, batch.entry_start,
-                              batch.entry_first_pos, batch.slots, self.a_log, self.dt_bias, self.kv_heads, self.dim,
-                              self.heads, self.vdim, b_col, b_col + self.heads, UNIT_EPS, qkv, beta, decay, entries)
+                              batch.entry_first_pos, batch.slots, self.a_log if plain else None,
+                              self.dt_bias if plain else None, self.kv_heads, self.dim, self.heads, self.vdim, b_col,
+                              a_col if plain else -1, UNIT_EPS, qkv, beta, decay if plain else None, entries)
+        if not plain:
+            raw = proj[:, a_col:a_col + self.decay_rows]
+            if self.decay_rank:
+                raw = self._second_step(raw, self.w_a2, torch.float32)
+            kernels.channel_decay(raw, self.a_log, self.dt_bias, self.heads, self.dim if self.per_channel else 1,
+                                  rows[:, self.channels:] if self.per_channel else decay)
         o = torch.empty((tokens, self.vw), **f32)
         kernels.delta_rule(qkv, beta, decay, state, batch.entry_start, batch.entry_first_pos, batch.slots,
-                           self.kv_heads, self.dim, self.heads, self.vdim, o, entries, short_entries=batch.all_single)
+                           self.kv_heads, self.dim, self.heads, self.vdim, o, entries, short_entries=batch.all_single,
+                           channel_decay_col=self.channels if self.per_channel else -1)
+        gate = proj[:, g_col:g_col + self.gate_rows]
+        if self.gate_rank:
+            gate = self._second_step(gate, self.w_g2, self.runtime.dtype)
         gated = self.runtime.empty((tokens, self.vw))
-        kernels.head_norm_gate(o, self.norm, proj[:, g_col:g_col + self.vw], True, self.eps, self.heads, self.vdim, gated)
-        linear(gated, self.w_o, None, residual, accumulate=True)
+        kernels.head_norm_gate(o, self.norm, gate, self.gate_kind, self.eps, self.heads, self.vdim, gated)
+        linear(gated, self.w_o, None, residual, accumulate=accumulate)
+
+
+class MatrixMemory(Mixer):
+    """``params``: ``hidden``, ``heads``, ``dim``, ``vdim``, ``gate_cap``, ``eps`` (of the read-out's norm), ``name``;
+    tensors ``<name>.q | k | v | g | o | norm | i | i.b | f | f.b``."""
+
+    can_overwrite = True
+
+    def __init__(self, spec: PartSpec, prefix: str, runtime):
+        super().__init__(spec, prefix, runtime)
+        p = spec.params
+        self.hidden, self.heads, self.dim, self.vdim = int(p["hidden"]), int(p["heads"]), int(p["dim"]), int(p["vdim"])
+        self.cap, self.eps = float(p["gate_cap"]), float(p["eps"])
+        self.qk, self.vw = self.heads * self.dim, self.heads * self.vdim
+        self.w_in = self.b_in = self.w_o = self.norm = None
+
+    @classmethod
+    def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
+        p = spec.params
+        base = f"{prefix}{p['name']}."
+        hidden, heads = int(p["hidden"]), int(p["heads"])
+        qk, vw = heads * int(p["dim"]), heads * int(p["vdim"])
+        return [TensorSpec(base + "q", (qk, hidden), MATRIX), TensorSpec(base + "k", (qk, hidden), MATRIX),
+                TensorSpec(base + "v", (vw, hidden), MATRIX), TensorSpec(base + "g", (vw, hidden), MATRIX),
+                TensorSpec(base + "o", (hidden, vw), MATRIX), TensorSpec(base + "norm", (vw,), VECTOR, "one_plus_normal"),
+                TensorSpec(base + "i", (heads, hidden), MATRIX), TensorSpec(base + "i.b", (heads,), VECTOR, std=0.5),
+                TensorSpec(base + "f", (heads, hidden), MATRIX), TensorSpec(base + "f.b", (heads,), VECTOR, std=0.5)]
+
+    @classmethod
+    def declare_cache(cls, spec: PartSpec):
+        p = spec.params
+        return None, StateSpec((kernels.memory_state_floats(int(p["heads"]), int(p["dim"]), int(p["vdim"])),), torch.float32)
+
+    @classmethod
+    def check_supported(cls, spec: PartSpec, dtype: torch.dtype) -> None:
+        p = spec.params
+        if int(p["dim"]) > kernels.RECURRENT_MAX_KEY_DIM:
+            raise UnsupportedError(f"matrix_memory: a key width of {p['dim']} is above the kernel's limit of "
+                                   f"{kernels.RECURRENT_MAX_KEY_DIM}")
+        if not float(p["gate_cap"]) > 0.0:
+            raise InvalidArgumentError(f"matrix_memory: gate_cap is {p['gate_cap']!r}; it must be above 0")
+
+    def load(self, tensors: Dict[str, torch.Tensor]) -> None:
+        base = f"{self.prefix}{self.spec.params['name']}."
+        self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", "g", "i", "f")])   # one product for all that reads h
+        bias = torch.zeros(self.w_in.shape[0], dtype=torch.float32, device=self.w_in.device)
+        bias[-2 * self.heads:-self.heads] = tensors[base + "i.b"].float()
+        bias[-self.heads:] = tensors[base + "f.b"].float()
+        self.b_in = bias
+        self.w_o, self.norm = tensors[base + "o"], tensors[base + "norm"]
+
+    def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
+        tokens, entries = residual.shape[0], batch.num_entries
+        proj = torch.empty((tokens, self.w_in.shape[0]), dtype=torch.float32, device=residual.device)
+        linear(h, self.w_in, self.b_in, proj)              # 32-bit from the product's sums on
+        k_col, v_col = self.qk, 2 * self.qk
+        g_col = v_col + self.vw
+        i_col = g_col + self.vw
+        o = torch.empty((tokens, self.vw), dtype=torch.float32, device=residual.device)
+        kernels.memory_rule(proj, 0, k_col, v_col, i_col, i_col + self.heads, self.dim ** -0.5, self.cap, state,
+                            batch.entry_start, batch.entry_first_pos, batch.slots, self.dim, self.heads, self.vdim, o,
+                            entries, short_entries=batch.all_single)
+        gated = self.runtime.empty((tokens, self.vw))
+        kernels.head_norm_gate(o, self.norm, proj[:, g_col:g_col + self.vw], "sigmoid", self.eps, self.heads, self.vdim, gated)
+        linear(gated, self.w_o, None, residual, accumulate=accumulate)
 
 
 class Wkv(Mixer):
@@ -366,6 +494,7 @@ class SelectiveScan(Mixer):
 
 
 register_mixer("gated_delta", GatedDelta)
+register_mixer("matrix_memory", MatrixMemory)
 register_mixer("decay_attention", DecayAttention)
 register_mixer("selective_scan", SelectiveScan)
 register_mixer("wkv", Wkv)
