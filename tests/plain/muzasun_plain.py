@@ -170,13 +170,24 @@ def gated_feed_forward(h, w, pre):
     return (silu(h @ w[pre + "gate"].T) * (h @ w[pre + "up"].T)) @ w[pre + "down"].T
 
 
-def mixture_of_experts(h, w, pre, m):
-    """Sigmoid scores; the best ``top`` experts, each fed the token times its score; a shared expert for every token."""
+def route(scores, top):
+    """The ``top`` experts with the largest scores, the lower id among equals."""
+    return sorted(range(len(scores)), key=lambda e: (-scores[e], e))[:top]
+
+
+def mixture_of_experts(h, w, pre, m, gaps=None):
+    """Sigmoid scores; the best ``top`` experts, each fed the token times its score; a shared expert for every token.
+    ``gaps`` (a list) receives, per token, how far the router's logit of the last chosen expert lies above the best one
+    left out (infinite where every expert is chosen)."""
     experts, top = m["router"]["experts"], m["router"]["top"]
-    scores = sigmoid(h @ w[pre + "router"].T)
+    logits = h @ w[pre + "router"].T
+    scores = sigmoid(logits)
     out = np.zeros((h.shape[0], w[pre + "e0.down"].shape[0]))
+    if gaps is not None:
+        ranked = -np.sort(-logits, axis=1)
+        gaps.append(ranked[:, top - 1] - ranked[:, top] if top < experts else np.full(h.shape[0], np.inf))
     for t in range(h.shape[0]):
-        chosen = sorted(range(experts), key=lambda e: (-scores[t, e], e))[:top]
+        chosen = route(scores[t], top)
         for e in chosen:
             out[t] += gated_feed_forward(scores[t, e] * h[t][None, :], w, f"{pre}e{e}.")[0]
     if m.get("shared"):
@@ -184,16 +195,17 @@ def mixture_of_experts(h, w, pre, m):
     return out
 
 
-def feed_forward(h, w, pre, m):
+def feed_forward(h, w, pre, m, gaps=None):
     if m is None:
         return 0.0
     if m["kind"] == "dense":
         return gated_feed_forward(h, w, pre)
-    return mixture_of_experts(h, w, pre, m)
+    return mixture_of_experts(h, w, pre, m, gaps)
 
 
-def forward(cfg, w, tokens, layers_out=None):
-    """Logits [T, vocab] of one sequence; ``layers_out`` (a list) receives the stream after every layer."""
+def forward(cfg, w, tokens, layers_out=None, gaps=None):
+    """Logits [T, vocab] of one sequence; ``layers_out`` (a list) receives the stream after every layer, ``gaps`` every
+    mixture's routing margins (see :func:`mixture_of_experts`)."""
     eps, mult = cfg["norm"]["eps"], cfg.get("residual_mult", 1.0)
     x = w["embed"][np.asarray(tokens)]
     v_first = None
@@ -211,7 +223,7 @@ def forward(cfg, w, tokens, layers_out=None):
             mixed = channel_delta_mixer(h, w, pre + "mix.", m, eps)
         else:
             raise ValueError(f"layer {index}: unknown type {kind!r}")
-        fed = feed_forward(dynamic_tanh(x, w, pre + "norm2"), w, pre + "mlp.", layer.get("mlp")) \
+        fed = feed_forward(dynamic_tanh(x, w, pre + "norm2"), w, pre + "mlp.", layer.get("mlp"), gaps) \
             if layer.get("mlp") is not None else 0.0
         x = x + mult * (mixed + fed)
         if layers_out is not None:

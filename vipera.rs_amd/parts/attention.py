@@ -124,6 +124,9 @@ class Attention(Mixer):
                       TensorSpec(base + names["k_norm"], (hd if per_head else kv,), VECTOR, "one_plus_normal")]
         if p.get("value_mix"):
             specs.append(TensorSpec(base + names["value_mix"], (), VECTOR, std=0.3))
+        elif "value_mix" in (p.get("tensors") or {}):
+            # a layer of a design that has the number but does not blend here: a folder may hold it all the same
+            specs.append(TensorSpec(base + names["value_mix"], (), VECTOR, std=0.3, optional=True))
         if p.get("gate"):
             specs.append(TensorSpec(base + names["g"], (int(p["heads"]) * vd, hidden), MATRIX))
         return specs
