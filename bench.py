@@ -106,7 +106,7 @@ def main() -> int:
                         help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
                              "pair of GPU events around every kernel launch, and add the microseconds of each class of "
                              "kernel to the line (split_decode_us, split_prefill_us)")
-    parser.add_argument("--design", default="", choices=["", "gilidra", "zulesun"],
+    parser.add_argument("--design", default="", choices=["", "gilidra", "zulesun", "muzasun"],
                         help="instead of the headline measurement: prefill and decode of this design at layer sizes that "
                              "resemble a real model's (--size), beside the dense Qwen2 decoder of the same width, depth and "
                              "active feed-forward width, each with the time of every class of kernel")
@@ -417,6 +417,32 @@ def zulesun_shape(z):
             "embedding": {"scale": z["width"] ** 0.5}, "token_side": {"dim": 64}, "layers": layers}
 
 
+def muzasun_shape(z):
+    """A Muzasun configuration of sizes ``z``: attention that blends values across layers, twice the matrix memory, the
+    delta rule with a decay per key channel, and so on; a dense feed-forward beside the attention layers and a mixture of
+    experts with a shared expert beside the others."""
+    heads = z["heads"]
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"], "top": z["top"]},
+           "shared": {"ff": z["ff"]}}
+    dense = {"kind": "dense", "ff": z["top"] * z["ff"]}
+    attention = {"heads": heads, "kv_heads": max(1, heads // 4), "dim": z["dim"], "vdim": z["dim"],
+                 "rot": {"base": 1e6, "dims": z["dim"] // 2}, "scale": z["dim"] ** -0.5, "v_mix": True}
+    memory = {"heads": heads, "dim": z["dim"], "vdim": z["dim"], "gate_cap": 15.0}
+    delta = {"heads": z["delta_heads"], "kv_heads": z["delta_kv"], "dim": 128, "vdim": 128, "conv": 4,
+             "decay_rank": 64, "gate_rank": 64}
+    layers = []
+    for index in range(z["layers"]):
+        kind = index % 5
+        if kind in (0, 4):
+            layers.append({"type": "attention", "mixer": attention, "mlp": dense})
+        elif kind == 3:
+            layers.append({"type": "channel_delta", "mixer": delta, "mlp": moe})
+        else:
+            layers.append({"type": "mlstm", "mixer": memory, "mlp": moe})
+    return {"architecture": "Muzasun", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "residual_mult": 0.5, "logit_scale": 0.5, "layers": layers}
+
+
 def dense_shape(z):
     """The dense Qwen2 decoder of the same width, depth, heads and active feed-forward width."""
     return dict(QWEN25_7B, num_hidden_layers=z["layers"], hidden_size=z["width"], num_attention_heads=z["heads"],
@@ -445,9 +471,11 @@ def design_comparison(args) -> int:
     largest = max(batches)
     gen = torch.Generator().manual_seed(0)
     out = {}
-    # Gilidra beside the dense decoder; Zulesun beside Gilidra, the engine's other decoder of recurrences, attention
-    # over a part of the positions and mixtures of experts, and beside the dense decoder
+    # Gilidra beside the dense decoder; Zulesun and Muzasun each beside Gilidra, the engine's other decoder of
+    # recurrences and mixtures of experts behind Dynamic Tanh norms, and beside the dense decoder
     runs = ((("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))) if args.design == "gilidra" else
+            (("muzasun", muzasun_shape(z)), ("gilidra", gilidra_shape(z)), ("dense", dense_shape(z)))
+            if args.design == "muzasun" else
             (("zulesun", zulesun_shape(z)), ("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))))
     for name, shape in runs:
         config = config_from_dict(shape)

@@ -2,6 +2,8 @@
 
 The file lists the layers one by one: ``layers[i]`` has ``type`` (which mixer: ``attention``, ``mlstm`` or
 ``channel_delta``), ``mixer`` (its sizes and constants) and ``mlp`` (``kind`` ``dense`` or ``moe``, or null for none).
+The inner sizes of the delta rule's two-step projections are those of the folder's tensors; ``decay_rank`` and
+``gate_rank`` in its ``mixer`` may state them.
 Beside the list stand ``vocab``, ``width``, ``norm.eps``, ``residual_mult`` and ``logit_scale``.  Every layer is a
 parallel block with a Dynamic Tanh norm of its own in front of each sublayer, both of the same stream:
 ``x += residual_mult * (mixer(norm1(x)) + mlp(norm2(x)))``; the last layer is followed by such a norm too.  Among the
@@ -181,7 +183,10 @@ class MuzasunConfig(ModelConfig):
                 mixer = PartSpec("gated_delta", {
                     "hidden": self.width, "heads": int(m["heads"]), "kv_heads": int(m["kv_heads"]), "dim": int(m["dim"]),
                     "vdim": int(m["vdim"]), "conv": int(m["conv"]), "eps": self.eps, "decay": "channel",
-                    "decay_rank": -1, "gate_rank": -1, "gate": "sigmoid", "name": "mix"})
+                    # the two-step projections' inner sizes are the folder's tensors' unless the file gives them
+                    # (a model of random weights has no folder to ask)
+                    "decay_rank": int(m.get("decay_rank") or -1), "gate_rank": int(m.get("gate_rank") or -1),
+                    "gate": "sigmoid", "name": "mix"})
             specs.append(LayerSpec("parallel", mixer, self._ffn(layer.get("mlp")), self._norm("norm1"), self._norm("norm2"),
                                    position, f"l{index}.", params={"residual_mult": self.residual_mult}))
         return specs
