@@ -134,6 +134,12 @@ __device__ __forceinline__ float dpp_add(float v) {
   return v + __int_as_float(moved);
 }
 
+// Lane l of a row of 16 gets the value of lane l - N of its row, or `edge` where the row has no such lane.
+template <int N>
+__device__ __forceinline__ float row_shifted(float v, float edge) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(v), 0x110 + N, 0xF, 0xF, false));
+}
+
 // The sum over the 16 lanes of a row, in every lane: neighbours, pairs of neighbours, the halves of eight, the eights.
 __device__ __forceinline__ float row_sum16(float v) {
   v = dpp_add<0xB1>(v);     // quad_perm [1, 0, 3, 2]
@@ -744,12 +750,38 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
     __syncthreads();
     if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
     const int count = min(REC_BLOCK, end - t0);
-    for (int j = 0; j < count; ++j) {
+    // The block's running maxima in closed form, so that no exponential waits for the token before it: with F_j the sum
+    // of the forget gates' logarithms up to token j of the block and m0 the maximum the block starts from,
+    // m_j = F_j + max(m0, max over l <= j of (li_l - F_l)).  Lane l of every row of sixteen works out token l & 15: two
+    // scans along the row (sum, then maximum), its maximum and its neighbour's before it, and from those its three
+    // exponentials; the token loop fetches them by lane.  Which sequence of maxima is used does not change the result
+    // beyond rounding, as long as S, n and the floor of the denominator use the same one; the sequence here is one fixed
+    // function of the block's gates and m0.
+    float keep_j, take_j, floor_j, m_j;
+    {
+      const int jj = lane & (REC_BLOCK - 1);
+      const float li_j = gates[jj][0], lf_j = gates[jj][1];
+      float F = lf_j;
+      F += row_shifted<1>(F, 0.f);
+      F += row_shifted<2>(F, 0.f);
+      F += row_shifted<4>(F, 0.f);
+      F += row_shifted<8>(F, 0.f);
+      float p = li_j - F;
+      p = fmaxf(p, row_shifted<1>(p, -INFINITY));
+      p = fmaxf(p, row_shifted<2>(p, -INFINITY));
+      p = fmaxf(p, row_shifted<4>(p, -INFINITY));
+      p = fmaxf(p, row_shifted<8>(p, -INFINITY));
+      m_j = F + fmaxf(m, p);
+      const float m_before = row_shifted<1>(m_j, m);      // the first token's: what the block starts from
+      keep_j = expf(lf_j + m_before - m_j), take_j = expf(li_j - m_j), floor_j = expf(-m_j);
+    }
+    m = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m_j), count - 1));
+    float tops = 0.f, unders = 0.f;
+    auto token = [&](int j) {
       const float* row = rows + j * ROW;
-      const float li = gates[j][0], lf = gates[j][1], val = row[2 * DP + wave];
-      const float m_new = fmaxf(lf + m, li);
-      const float a = expf(lf + m - m_new), b = expf(li - m_new);
-      m = m_new;
+      const float val = row[2 * DP + wave];
+      const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(keep_j), j));
+      const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(take_j), j));
       float num = 0.f, den = 0.f;
 #pragma unroll
       for (int i = 0; i < Q; ++i) {
@@ -761,8 +793,17 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
       }
       num = wave_total(num);
       den = wave_total(den);
-      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = num / (fmaxf(fabsf(den), expf(-m)) + 1e-6f);
+      tops = lane == j ? num : tops;        // lane j keeps token j's two sums: the division waits for the block's end
+      unders = lane == j ? den : unders;
+    };
+    if (count == REC_BLOCK) {      // a whole block: every lane index and LDS offset is a constant
+#pragma unroll
+      for (int j = 0; j < REC_BLOCK; ++j) token(j);
+    } else {
+      for (int j = 0; j < count; ++j) token(j);
     }
+    if (live && lane < count)     // lane j < 16 also holds token j's floor
+      out[((long long)(t0 + lane) * heads + h) * vdim + v] = tops / (fmaxf(fabsf(unders), floor_j) + 1e-6f);
   }
 #pragma unroll
   for (int i = 0; i < Q; ++i)
