@@ -135,6 +135,23 @@ def test_heads_normed_one_by_one_and_values_blended(dtype):
     assert not got[:, :heads + kv_heads, dim:].any() and not got[:, heads + kv_heads:, vdim:].any()     # zeros in the padding
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_two_norms_of_the_same_rows_in_one_launch(dtype):
+    from vipera_rs_amd.ops import kernels
+
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((7, 50)) * 2.0
+    dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.float32, device="cuda")
+    norms = [(np.array([0.7 + k]), 1 + 0.1 * rng.standard_normal(50), 0.1 * rng.standard_normal(50)) for k in range(2)]
+    outs = [torch.empty((7, 50), dtype=dtype, device="cuda") for _ in range(2)]
+    kernels.dyt_pair(dev(x), *[tuple(dev(t) for t in norm) for norm in norms], *outs)
+    for (alpha, weight, bias), out in zip(norms, outs):
+        single = torch.empty_like(out)
+        kernels.dyt(dev(x), dev(alpha), dev(weight), dev(bias), single)
+        assert torch.equal(out, single)                  # the same bits as the norm alone
+        assert rel_err(out.float().cpu().numpy(), np.tanh(alpha * x) * weight + bias) < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
 # --- each mechanism alone, as a model of one layer -------------------------------------------------------------------
 ONE_LAYER = {
     # the matrix memory at every register layout of its two kernels (1 to 16 key channels a lane)

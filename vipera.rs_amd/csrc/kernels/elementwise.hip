@@ -501,6 +501,41 @@ extern "C" int vk_dyt(const float* x, const float* alpha, const float* weight, c
   return 0;
 }
 
+// Two Dynamic Tanh norms of the same rows in one launch (a layer whose two sublayers each read a norm of their own):
+// out_k = tanh(alpha_k * x) * weight_k + bias_k for k = 1, 2; every element of x is read once.
+template <typename TO>
+__global__ __launch_bounds__(256) void dyt_pair_kernel(const float* __restrict__ x, const float* __restrict__ alpha1,
+                                                       const float* __restrict__ weight1, const float* __restrict__ bias1,
+                                                       TO* __restrict__ out1, const float* __restrict__ alpha2,
+                                                       const float* __restrict__ weight2, const float* __restrict__ bias2,
+                                                       TO* __restrict__ out2, int width) {
+  const size_t base = (size_t)blockIdx.x * width;
+  const float a1 = alpha1[0], a2 = alpha2[0];
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    const float v = x[base + c];
+    out1[base + c] = from_float<TO>(fmaf(tanhf(a1 * v), weight1[c], bias1[c]));
+    out2[base + c] = from_float<TO>(fmaf(tanhf(a2 * v), weight2[c], bias2[c]));
+  }
+}
+
+extern "C" int vk_dyt_pair(const float* x, const float* alpha1, const float* weight1, const float* bias1, void* out1,
+                           const float* alpha2, const float* weight2, const float* bias2, void* out2, int out_dtype,
+                           int num_rows, int width, void* stream) {
+  if (num_rows <= 0) return 0;
+  if (width <= 0) return VK_BAD_ARGUMENT;
+  hipStream_t s = (hipStream_t)stream;
+  if (out_dtype == DT_F32)
+    dyt_pair_kernel<float><<<num_rows, 256, 0, s>>>(x, alpha1, weight1, bias1, (float*)out1, alpha2, weight2, bias2,
+                                                    (float*)out2, width);
+  else if (out_dtype == DT_BF16)
+    dyt_pair_kernel<bf16_t><<<num_rows, 256, 0, s>>>(x, alpha1, weight1, bias1, (bf16_t*)out1, alpha2, weight2, bias2,
+                                                     (bf16_t*)out2, width);
+  else
+    return VK_BAD_ARGUMENT;
+  VK_LAUNCH_CHECK();
+  return 0;
+}
+
 // x *= factor, elementwise, 32-bit.
 __global__ void scale_kernel(float* __restrict__ x, float factor, long long count) {
   const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -910,6 +910,24 @@ def dyt(x: torch.Tensor, alpha: torch.Tensor, weight: torch.Tensor, bias: torch.
                _stream()), "dyt")
 
 
+def dyt_pair(x: torch.Tensor, first, second, out1: torch.Tensor, out2: torch.Tensor) -> None:
+    """Two Dynamic Tanh norms of the same rows in one launch: ``out_k = tanh(alpha_k * x) * weight_k + bias_k``; ``first``
+    and ``second`` are ``(alpha, weight, bias)`` as :func:`dyt` takes them."""
+    width = x.shape[1]
+    _need(x.dim() == 2 and x.dtype == torch.float32 and x.is_contiguous(), "dyt_pair: x must be contiguous float32 [tokens, width]")
+    for alpha, weight, bias in (first, second):
+        _dev(x, alpha, weight, bias)
+        _need(alpha.dtype == torch.float32 and alpha.numel() == 1, "dyt_pair: alpha must be one float32")
+        for name, t in (("weight", weight), ("bias", bias)):
+            _need(t.dtype == torch.float32 and t.numel() == width and t.is_contiguous(), f"dyt_pair: {name} must be float32 [width]")
+    _dev(out1, out2)
+    _need(out1.shape == x.shape and out2.shape == x.shape and out1.is_contiguous() and out2.is_contiguous()
+          and out1.dtype == out2.dtype, "dyt_pair: outputs")
+    fn = _fn("elementwise", "vk_dyt_pair", [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _p])
+    _status(fn(_ptr(x), _ptr(first[0]), _ptr(first[1]), _ptr(first[2]), _ptr(out1), _ptr(second[0]), _ptr(second[1]),
+               _ptr(second[2]), _ptr(out2), _dt(out1, "out"), x.shape[0], width, _stream()), "dyt_pair")
+
+
 def scale_(x: torch.Tensor, factor: float) -> None:
     """``x *= factor`` (32-bit, in place)."""
     _dev(x)

@@ -29,7 +29,7 @@ LAUNCHERS = (
     "dyt", "scale_", "tanh", "decay_", "delta_prepare", "delta_rule", "wkv_rule", "token_shift", "head_norm_gate",
     "latent_kv_write", "latent_q_rotate", "head_linear", "moe_route", "moe_experts",
     "rmsnorm_add", "axpby", "activation", "whole_norm_pack", "head_unpack_gate", "decay_rule", "gated_norm",
-    "causal_conv", "selective_scan", "scan_prepare", "head_norm_pack", "channel_decay", "memory_rule",
+    "causal_conv", "selective_scan", "scan_prepare", "head_norm_pack", "channel_decay", "memory_rule", "dyt_pair",
 )
 
 

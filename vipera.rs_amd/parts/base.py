@@ -116,6 +116,10 @@ class Norm(Part):
                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_with(self, other: "Norm", x: torch.Tensor):
+        """``(self.forward(x), other.forward(x))``: two norms of the same rows; a kind that can runs them as one launch."""
+        return self.forward(x), other.forward(x)
+
     def handoff(self, tokens: int) -> Optional[NormHandoff]:
         """A :class:`NormHandoff` for ``tokens`` rows if this norm can be split between its neighbours, else None."""
         return None

@@ -128,8 +128,11 @@ class ParallelBlock(Block):
                 part.load(tensors)
 
     def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
-        h = self.norm.forward(x)
-        h_ffn = self.ffn_norm.forward(x) if self.ffn_norm is not None else h
+        if self.ffn_norm is not None and type(self.ffn_norm) is type(self.norm):
+            h, h_ffn = self.norm.forward_with(self.ffn_norm, x)       # both norms of the same rows: one launch
+        else:
+            h = self.norm.forward(x)
+            h_ffn = self.ffn_norm.forward(x) if self.ffn_norm is not None else h
         if self.mult == 1.0:
             # both sublayers add into the 32-bit residual; neither reads it after the norms, so their order does not matter
             self.mixer.forward(h, batch, cache, state, self.position, x, reads_only)
