@@ -372,6 +372,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
   const bool live = v < vdim;
   const int kh = h / (heads / kv_heads);
   const int start = entry_start[e], end = entry_start[e + 1];
+  if (start >= end) return;      // the whole workgroup
   float* mine = state + (long long)slots[e] * state_stride + ((long long)h * value_pad + v) * key_pad + d0;
   const bool fresh = entry_first[e] == 0, kept = v < value_pad;
   float S[Q];
@@ -390,30 +391,31 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
     }
     plan[i] = within < 0 ? -1 : (j << 24) | within;
   }
-  float held[LOADS], held_gate = 0.f;
+  // A fetch only issues loads, every thread the same number of them and none inside a branch, from addresses that
+  // exist whatever the block holds (the entry's last token stands in for tokens past its end, which are never worked
+  // on; column 0 for numbers that are always zero).  A loaded number is first used when it is stored into LDS, a block
+  // later, so that nothing waits for memory before the block in between has been worked on.
+  float held[LOADS], held_gate;
+  const float* gate_src = ((tid & 1) && !CH ? decay : beta) + h;
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
-      // a token past the entry's end is never worked on: its address is clamped, its value does not matter
       const int t = min(t0 + (plan[i] >> 24 & 127), end - 1);
-      const float loaded = qkv[(long long)t * ldq + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
-      held[i] = plan[i] < 0 ? 0.f : loaded;
+      held[i] = qkv[(long long)t * ldq + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
     }
-    if (tid < 2 * REC_BLOCK) {
-      const int t = min(t0 + (tid >> 1), end - 1);
-      held_gate = ((tid & 1) && !CH ? decay : beta)[(long long)t * heads + h];
-    }
+    held_gate = gate_src[(long long)min(t0 + ((tid >> 1) & (REC_BLOCK - 1)), end - 1) * heads];
   };
   fetch(start);
   for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
     __syncthreads();     // the block before has been read
 #pragma unroll
     for (int i = 0; i < LOADS; ++i)
-      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = plan[i] < 0 ? 0.f : held[i];
     if (tid < 2 * REC_BLOCK) gates[tid >> 1][tid & 1] = held_gate;
     __syncthreads();
-    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    fetch(min(t0 + REC_BLOCK, end - 1));
     const int count = min(REC_BLOCK, end - t0);
+    float outs = 0.f;      // lane j of every row: its row's part of token j's read-out, which nothing waits for
     for (int j = 0; j < count; ++j) {
       const float* row = rows + j * ROW;
       const float b = gates[j][0], g = gates[j][1], val = row[VOFF + wave];
@@ -436,9 +438,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void delta_scan_kernel(
         S[i] = fmaf(kk[i], u, S[i]);
         o = fmaf(S[i], qq[i], o);
       }
-      o = wave_total(o);
-      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * vdim + v] = o;
+      o = row_sum16(o);
+      outs = (lane & (REC_BLOCK - 1)) == j ? o : outs;
     }
+    outs += __shfl_xor(outs, 16, 64);     // (row 0 + row 1) + (row 2 + row 3), in every row
+    outs += __shfl_xor(outs, 32, 64);
+    if (live && lane < count) out[((long long)(t0 + lane) * heads + h) * vdim + v] = outs;
   }
   if (kept) {
 #pragma unroll
@@ -462,6 +467,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
   const int v0 = blockIdx.z * SCAN_COLS, col_v = v0 + wave;
   const bool live = col_v < dim;
   const int start = entry_start[e], end = entry_start[e + 1];
+  if (start >= end) return;      // the whole workgroup
   float* mine = state + (long long)slots[e] * state_stride + ((long long)h * value_pad + col_v) * key_pad + d0;
   const bool fresh = entry_first[e] == 0, kept = col_v < value_pad;
   float S[Q], U[Q];
@@ -479,6 +485,8 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
     const int d = kind < 3 ? col - kind * DP : v0 + col - 3 * DP;
     plan[i] = (x < COUNT && d < dim) ? (kind << 28) | (j << 21) | d : -1;
   }
+  // A fetch only issues loads, the same number in every thread and none inside a branch, from addresses that exist
+  // whatever the block holds; a loaded number is first used when it is stored into LDS, a block later.
   float held[LOADS];
   auto fetch = [&](int t0) {
 #pragma unroll
@@ -486,23 +494,25 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
       const int kind = plan[i] >> 28 & 3, d = plan[i] < 0 ? 0 : plan[i] & 0x1FFFFF;
       const long long t = min(t0 + (plan[i] >> 21 & 127), end - 1);
       const float* base = kind == 0 ? r + t * ldr : kind == 1 ? k + t * ldk : kind == 2 ? wraw + t * ldw : v + t * ldv;
-      float loaded = base[h * dim + d];
-      if (!decayed) {      // the same for every thread: the caller has not turned wraw into the decay yet
-        const float shift = w0[h * dim + d];
-        loaded = kind == 2 ? expf(-expf(loaded + shift)) : loaded;
-      }
-      held[i] = plan[i] < 0 ? 0.f : loaded;
+      held[i] = base[h * dim + d];
     }
   };
   fetch(start);
   for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i)
-      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+    for (int i = 0; i < LOADS; ++i) {
+      float value = held[i];
+      if (!decayed) {      // the same for every thread: the caller has not turned wraw into the decay yet
+        const float shift = w0[h * dim + (plan[i] < 0 ? 0 : plan[i] & 0x1FFFFF)];
+        value = (plan[i] >> 28 & 3) == 2 ? expf(-expf(value + shift)) : value;
+      }
+      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = plan[i] < 0 ? 0.f : value;
+    }
     __syncthreads();
-    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    fetch(min(t0 + REC_BLOCK, end - 1));
     const int count = min(REC_BLOCK, end - t0);
+    float outs = 0.f;      // lane j of every row: its row's part of token j's read-out, which nothing waits for
     for (int j = 0; j < count; ++j) {
       const float* row = rows + j * ROW;
       const float val = row[3 * DP + wave];
@@ -513,9 +523,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void wkv_scan_kernel(
         o = fmaf(fmaf(U[i], kv, S[i]), row[d0 + i], o);
         S[i] = fmaf(row[2 * DP + d0 + i], S[i], kv);
       }
-      o = wave_total(o);
-      if (live && lane == 0) out[((long long)(t0 + j) * heads + h) * dim + col_v] = o;
+      o = row_sum16(o);
+      outs = (lane & (REC_BLOCK - 1)) == j ? o : outs;
     }
+    outs += __shfl_xor(outs, 16, 64);     // (row 0 + row 1) + (row 2 + row 3), in every row
+    outs += __shfl_xor(outs, 32, 64);
+    if (live && lane < count) out[((long long)(t0 + lane) * heads + h) * dim + col_v] = outs;
   }
   if (kept) {
 #pragma unroll
@@ -681,23 +694,42 @@ __global__ __launch_bounds__(256) void memory_rule_kernel(
   }
 }
 
+// The gates' logarithms of a step's tokens, in place: proj[t, i_col + h] <- li, proj[t, f_col + h] <- lf.  A prompt's
+// recurrence reads them a block of tokens at a time and takes no tanh or logarithm itself.
+__global__ __launch_bounds__(256) void memory_gates_kernel(float* __restrict__ proj, long long ldp, int i_col, int f_col,
+                                                           int heads, float cap, long long count) {
+  const long long x = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (x >= count) return;
+  float* p = proj + x / heads * ldp + x % heads;
+  p[i_col] = log_gate(p[i_col], cap, false);
+  p[f_col] = log_gate(p[f_col], cap, true);
+}
+
 // Prompts' portions: the scan shape (a wave owns one value channel and its 64 lanes the key channels, eight waves to a
-// workgroup, tokens through LDS in blocks of 16 fetched a block ahead).  Every wave carries n and m itself.
+// workgroup, tokens through LDS in blocks of 16 fetched a block ahead).  Every wave carries n and m itself, but n . q
+// is the same number in all eight waves: each works it out for two of the block's tokens and leaves it in LDS.  Nothing
+// of a token's read-out goes back into the state, so S^T q is summed inside each row of sixteen lanes as the tokens
+// pass (lane j of a row keeps token j's) and across the four rows once per block.
 // An LDS row of a token: [q: 64Q | k: 64Q | v: 8]; the two gates' logarithms lie beside.  Grid (entries, heads, tiles).
+// The gates' columns of `proj` hold the logarithms li and lf already (memory_gates_kernel).
 template <int Q>
 __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
-    const float* __restrict__ proj, long long ldp, MemoryColumns col, float q_scale, float cap,
+    const float* __restrict__ proj, long long ldp, MemoryColumns col, float q_scale,
     float* __restrict__ state, long long state_stride, long long n_offset, long long m_offset,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first, const int* __restrict__ slots, int dim,
     int heads, int vdim, int key_pad, int value_pad, float* __restrict__ out) {
   constexpr int DP = 64 * Q, ROW = 2 * DP + SCAN_COLS, COUNT = REC_BLOCK * ROW, LOADS = (COUNT + SCAN_THREADS - 1) / SCAN_THREADS;
+  constexpr int PER_WAVE = REC_BLOCK / SCAN_COLS;     // tokens of a block whose n . q a wave works out
+  static_assert(PER_WAVE * SCAN_COLS == REC_BLOCK && REC_BLOCK == 16, "a block's tokens are a row of lanes, dealt to the waves");
   __shared__ float rows[COUNT];
   __shared__ float gates[REC_BLOCK][2];
+  __shared__ float dens[REC_BLOCK];
   const int e = blockIdx.x, h = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int d0 = lane * Q;
   const int v0 = blockIdx.z * SCAN_COLS, v = v0 + wave;
   const bool live = v < vdim;
   const int start = entry_start[e], end = entry_start[e + 1];
+  if (start >= end) return;      // the whole workgroup
   float* row0 = state + (long long)slots[e] * state_stride;
   float* mine = row0 + ((long long)h * value_pad + v) * key_pad + d0;
   float* my_n = row0 + n_offset + ((long long)h * gridDim.z + blockIdx.z) * key_pad + d0;
@@ -715,6 +747,7 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
   float m = fresh ? 0.f : m_old;
   // a block's fetch plan: token * 2^24 + the column inside the token's row of proj, or -1 for what is always zero
   int plan[LOADS];
+  unsigned is_q = 0;     // bit i: element i of this thread is a query's number
 #pragma unroll
   for (int i = 0; i < LOADS; ++i) {
     const int x = tid + i * SCAN_THREADS, j = x / ROW, c = x % ROW;
@@ -725,30 +758,32 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
       else if (v0 + c - 2 * DP < vdim) within = col.v + h * vdim + v0 + c - 2 * DP;
     }
     plan[i] = within < 0 ? -1 : (j << 24) | within;
+    is_q |= (unsigned)(c < DP) << i;
   }
-  float held[LOADS], held_gate = 0.f;
+  // A fetch only issues loads, every thread the same number of them and none inside a branch, from addresses that
+  // exist whatever the block holds (the entry's last token stands in for tokens past its end, column 0 for numbers that
+  // are always zero); what a loaded number becomes is decided when it is stored into LDS, a block later, so that
+  // nothing waits for memory before the block in between has been worked on.
+  float held[LOADS], held_gate;
+  const int gate_col = ((tid & 1) ? col.f : col.i) + h;
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int i = 0; i < LOADS; ++i) {
       const int t = min(t0 + (plan[i] >> 24 & 127), end - 1);
-      const float loaded = proj[(long long)t * ldp + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
-      const bool is_q = (tid + i * SCAN_THREADS) % ROW < DP;
-      held[i] = plan[i] < 0 ? 0.f : is_q ? loaded * q_scale : loaded;
+      held[i] = proj[(long long)t * ldp + (plan[i] < 0 ? 0 : plan[i] & 0xFFFFFF)];
     }
-    if (tid < 2 * REC_BLOCK) {
-      const int t = min(t0 + (tid >> 1), end - 1);
-      held_gate = log_gate(proj[(long long)t * ldp + ((tid & 1) ? col.f : col.i) + h], cap, tid & 1);
-    }
+    held_gate = proj[(long long)min(t0 + ((tid >> 1) & (REC_BLOCK - 1)), end - 1) * ldp + gate_col];
   };
   fetch(start);
   for (int t0 = start; t0 < end; t0 += REC_BLOCK) {
-    __syncthreads();     // the block before has been read
+    // the block before has been read: every wave has passed the barrier at its end
 #pragma unroll
     for (int i = 0; i < LOADS; ++i)
-      if (tid + i * SCAN_THREADS < COUNT) rows[tid + i * SCAN_THREADS] = held[i];
+      if (tid + i * SCAN_THREADS < COUNT)
+        rows[tid + i * SCAN_THREADS] = plan[i] < 0 ? 0.f : (is_q >> i & 1) ? held[i] * q_scale : held[i];
     if (tid < 2 * REC_BLOCK) gates[tid >> 1][tid & 1] = held_gate;
     __syncthreads();
-    if (t0 + REC_BLOCK < end) fetch(t0 + REC_BLOCK);
+    fetch(min(t0 + REC_BLOCK, end - 1));
     const int count = min(REC_BLOCK, end - t0);
     // The block's running maxima in closed form, so that no exponential waits for the token before it: with F_j the sum
     // of the forget gates' logarithms up to token j of the block and m0 the maximum the block starts from,
@@ -776,25 +811,30 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
       keep_j = expf(lf_j + m_before - m_j), take_j = expf(li_j - m_j), floor_j = expf(-m_j);
     }
     m = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m_j), count - 1));
-    float tops = 0.f, unders = 0.f;
+    float tops = 0.f;      // lane j of every row: its row's part of token j's S^T q
     auto token = [&](int j) {
       const float* row = rows + j * ROW;
       const float val = row[2 * DP + wave];
       const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(keep_j), j));
       const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(take_j), j));
-      float num = 0.f, den = 0.f;
+      float num = 0.f, qq[Q];
 #pragma unroll
       for (int i = 0; i < Q; ++i) {
-        const float bk = b * row[DP + d0 + i], qq = row[d0 + i];
+        const float bk = b * row[DP + d0 + i];
+        qq[i] = row[d0 + i];
         S[i] = fmaf(bk, val, a * S[i]);
         N[i] = fmaf(a, N[i], bk);
-        num = fmaf(S[i], qq, num);
-        den = fmaf(N[i], qq, den);
+        num = fmaf(S[i], qq[i], num);
       }
-      num = wave_total(num);
-      den = wave_total(den);
-      tops = lane == j ? num : tops;        // lane j keeps token j's two sums: the division waits for the block's end
-      unders = lane == j ? den : unders;
+      if (wave == j / PER_WAVE) {       // the whole wave or none of it
+        float den = 0.f;
+#pragma unroll
+        for (int i = 0; i < Q; ++i) den = fmaf(N[i], qq[i], den);
+        den = wave_total(den);
+        if (lane == 0) dens[j] = den;
+      }
+      num = row_sum16(num);
+      tops = (lane & (REC_BLOCK - 1)) == j ? num : tops;
     };
     if (count == REC_BLOCK) {      // a whole block: every lane index and LDS offset is a constant
 #pragma unroll
@@ -802,8 +842,12 @@ __global__ __launch_bounds__(SCAN_THREADS) void memory_scan_kernel(
     } else {
       for (int j = 0; j < count; ++j) token(j);
     }
-    if (live && lane < count)     // lane j < 16 also holds token j's floor
-      out[((long long)(t0 + lane) * heads + h) * vdim + v] = tops / (fmaxf(fabsf(unders), floor_j) + 1e-6f);
+    // the four rows' parts: (row 0 + row 1) + (row 2 + row 3) in every row, whichever it is
+    tops += __shfl_xor(tops, 16, 64);
+    tops += __shfl_xor(tops, 32, 64);
+    __syncthreads();     // every token's n . q is in LDS, and the block has been read
+    if (live && lane < count)     // lane j < 16 also holds token j's floor; the division waits for the block's end
+      out[((long long)(t0 + lane) * heads + h) * vdim + v] = tops / (fmaxf(fabsf(dens[lane]), floor_j) + 1e-6f);
   }
 #pragma unroll
   for (int i = 0; i < Q; ++i)
@@ -964,11 +1008,13 @@ extern "C" long long vk_memory_state_floats(int heads, int dim, int vdim) {
   return (long long)heads * (vk_recurrent_head_floats(dim, vdim) + tiles * 16 * rows_of(dim) + tiles);
 }
 
-extern "C" int vk_memory_rule(const float* proj, long long ldp, int q_col, int k_col, int v_col, int i_col, int f_col,
-                              float q_scale, float cap, float* state, long long state_stride, const int* entry_start,
-                              const int* entry_first, const int* slots, int dim, int heads, int vdim, float* out,
-                              int num_entries, int short_entries, void* stream) {
-  if (num_entries <= 0) return 0;
+// `proj` holds `num_tokens` rows.  Unless `short_entries` says that every entry is a single token, the gates' columns
+// of `proj` are overwritten with their logarithms.
+extern "C" int vk_memory_rule(float* proj, long long ldp, int num_tokens, int q_col, int k_col, int v_col, int i_col,
+                              int f_col, float q_scale, float cap, float* state, long long state_stride,
+                              const int* entry_start, const int* entry_first, const int* slots, int dim, int heads,
+                              int vdim, float* out, int num_entries, int short_entries, void* stream) {
+  if (num_entries <= 0 || num_tokens <= 0) return 0;
   if (heads < 1 || dim < 1 || vdim < 1 || !(cap > 0.f)) return VK_BAD_ARGUMENT;
   if (dim > 256 || heads > 65535 || ldp >= (1 << 24)) return VK_UNSUPPORTED_SIZE;
   if (min(min(q_col, k_col), min(v_col, min(i_col, f_col))) < 0) return VK_BAD_ARGUMENT;
@@ -979,9 +1025,11 @@ extern "C" int vk_memory_rule(const float* proj, long long ldp, int q_col, int k
   const long long m_offset = n_offset + (long long)heads * tiles * key_pad;
   const MemoryColumns col{q_col, k_col, v_col, i_col, f_col};
   if (!short_entries) {
+    const long long gates = (long long)num_tokens * heads;
+    memory_gates_kernel<<<(unsigned)((gates + 255) / 256), 256, 0, s>>>(proj, ldp, i_col, f_col, heads, cap, gates);
     dim3 scan_grid(num_entries, heads, (unsigned)tiles);
 #define VK_MEMORY_SCAN(Q)                                                                                            \
-  memory_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(proj, ldp, col, q_scale, cap, state, state_stride, n_offset, \
+  memory_scan_kernel<Q><<<scan_grid, SCAN_THREADS, 0, s>>>(proj, ldp, col, q_scale, state, state_stride, n_offset,     \
                                                            m_offset, entry_start, entry_first, slots, dim, heads, vdim, \
                                                            key_pad, value_pad, out)
     if (key_pad <= 64) VK_MEMORY_SCAN(1);

@@ -1077,7 +1077,8 @@ def memory_rule(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col: i
     ``S = exp(lf + m - m') S + exp(li - m') k v^T``, ``n`` likewise with ``k`` alone,
     ``o = S^T q / (max(|n . q|, exp(-m')) + 1e-6)``.  q, k (``heads * dim`` each), v (``heads * vdim``) and the raw gates
     (``heads`` each) are columns of the 32-bit ``proj`` from the given offsets on; q is multiplied by ``q_scale``.  State
-    rows hold :func:`memory_state_floats` floats; ``out`` 32-bit ``[tokens, heads * vdim]``."""
+    rows hold :func:`memory_state_floats` floats; ``out`` 32-bit ``[tokens, heads * vdim]``.  Unless ``short_entries``
+    (every entry is one token), the two gates' columns of ``proj`` are overwritten with ``li`` and ``lf``."""
     _dev(proj, state, entry_start, entry_first, slots, out)
     tokens = proj.shape[0]
     _need(proj.dim() == 2 and proj.dtype == torch.float32 and proj.stride(1) == 1, "memory_rule: proj")
@@ -1092,8 +1093,8 @@ def memory_rule(proj: torch.Tensor, q_col: int, k_col: int, v_col: int, i_col: i
     _need(cap > 0.0, "memory_rule: the gates' cap must be above 0")
     if dim > RECURRENT_MAX_KEY_DIM:
         raise UnsupportedError(f"memory_rule: a key width of {dim} is above the kernel's limit of {RECURRENT_MAX_KEY_DIM}")
-    fn = _fn("recurrent", "vk_memory_rule", [_p, _ll, _i, _i, _i, _i, _i, _f, _f, _p, _ll, _p, _p, _p, _i, _i, _i, _p, _i, _i, _p])
-    _status(fn(_ptr(proj), proj.stride(0), q_col, k_col, v_col, i_col, f_col, float(q_scale), float(cap), _ptr(state),
+    fn = _fn("recurrent", "vk_memory_rule", [_p, _ll, _i, _i, _i, _i, _i, _i, _f, _f, _p, _ll, _p, _p, _p, _i, _i, _i, _p, _i, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), tokens, q_col, k_col, v_col, i_col, f_col, float(q_scale), float(cap), _ptr(state),
                state.stride(0), _ptr(entry_start), _ptr(entry_first), _ptr(slots), dim, heads, vdim, _ptr(out),
                num_entries, 1 if short_entries else 0, _stream()), "memory_rule")
 
