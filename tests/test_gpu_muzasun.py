@@ -136,14 +136,17 @@ def test_heads_normed_one_by_one_and_values_blended(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_two_norms_of_the_same_rows_in_one_launch(dtype):
+@pytest.mark.parametrize("rows, width", [(7, 50), (5, 1100), (3, 4700), (300, 520)])
+def test_two_norms_of_the_same_rows_in_one_launch(rows, width, dtype):
+    """Few rows are spread over several workgroups each (a last part that is not full, more columns than one pass of
+    all parts covers); many rows are a workgroup each."""
     from vipera_rs_amd.ops import kernels
 
     rng = np.random.default_rng(4)
-    x = rng.standard_normal((7, 50)) * 2.0
+    x = rng.standard_normal((rows, width)) * 2.0
     dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.float32, device="cuda")
-    norms = [(np.array([0.7 + k]), 1 + 0.1 * rng.standard_normal(50), 0.1 * rng.standard_normal(50)) for k in range(2)]
-    outs = [torch.empty((7, 50), dtype=dtype, device="cuda") for _ in range(2)]
+    norms = [(np.array([0.7 + k]), 1 + 0.1 * rng.standard_normal(width), 0.1 * rng.standard_normal(width)) for k in range(2)]
+    outs = [torch.empty((rows, width), dtype=dtype, device="cuda") for _ in range(2)]
     kernels.dyt_pair(dev(x), *[tuple(dev(t) for t in norm) for norm in norms], *outs)
     for (alpha, weight, bias), out in zip(norms, outs):
         single = torch.empty_like(out)

@@ -474,7 +474,12 @@ extern "C" int vk_fill_normal(void* out, int dtype, long long count, unsigned lo
 
 // ---------------------------------------------------------------------------------------------
 // Dynamic Tanh: out = tanh(alpha * x) * weight + bias, elementwise (no mean, no variance); alpha is one number,
-// read from device memory.  x: 32-bit rows of `width`; rows (optional) selects them.
+// read from device memory.  x: 32-bit rows of `width`; rows (optional) selects them.  Grid (rows, parts of a row): a
+// step of few rows spreads each over several workgroups (dyt_parts), a tanh being the longest thing a thread does.
+static inline unsigned dyt_parts(int num_rows, int width) {
+  return num_rows >= 256 ? 1u : (unsigned)min(16, (width + 255) / 256);
+}
+
 template <typename TO>
 __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, const float* __restrict__ alpha,
                                                   const float* __restrict__ weight, const float* __restrict__ bias,
@@ -483,7 +488,8 @@ __global__ __launch_bounds__(256) void dyt_kernel(const float* __restrict__ x, c
   const float* src = x + (size_t)(rows ? rows[r] : r) * width;
   TO* dst = out + (size_t)r * width;
   const float a = alpha[0];
-  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = from_float<TO>(fmaf(tanhf(a * src[c]), weight[c], bias[c]));
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x)
+    dst[c] = from_float<TO>(fmaf(tanhf(a * src[c]), weight[c], bias[c]));
 }
 
 extern "C" int vk_dyt(const float* x, const float* alpha, const float* weight, const float* bias, const int* rows,
@@ -491,10 +497,11 @@ extern "C" int vk_dyt(const float* x, const float* alpha, const float* weight, c
   if (num_rows <= 0) return 0;
   if (width <= 0) return VK_BAD_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(num_rows, dyt_parts(num_rows, width));
   if (out_dtype == DT_F32)
-    dyt_kernel<float><<<num_rows, 256, 0, s>>>(x, alpha, weight, bias, rows, (float*)out, width);
+    dyt_kernel<float><<<grid, 256, 0, s>>>(x, alpha, weight, bias, rows, (float*)out, width);
   else if (out_dtype == DT_BF16)
-    dyt_kernel<bf16_t><<<num_rows, 256, 0, s>>>(x, alpha, weight, bias, rows, (bf16_t*)out, width);
+    dyt_kernel<bf16_t><<<grid, 256, 0, s>>>(x, alpha, weight, bias, rows, (bf16_t*)out, width);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
@@ -511,7 +518,7 @@ __global__ __launch_bounds__(256) void dyt_pair_kernel(const float* __restrict__
                                                        TO* __restrict__ out2, int width) {
   const size_t base = (size_t)blockIdx.x * width;
   const float a1 = alpha1[0], a2 = alpha2[0];
-  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < width; c += gridDim.y * blockDim.x) {
     const float v = x[base + c];
     out1[base + c] = from_float<TO>(fmaf(tanhf(a1 * v), weight1[c], bias1[c]));
     out2[base + c] = from_float<TO>(fmaf(tanhf(a2 * v), weight2[c], bias2[c]));
@@ -524,12 +531,13 @@ extern "C" int vk_dyt_pair(const float* x, const float* alpha1, const float* wei
   if (num_rows <= 0) return 0;
   if (width <= 0) return VK_BAD_ARGUMENT;
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(num_rows, dyt_parts(num_rows, width));
   if (out_dtype == DT_F32)
-    dyt_pair_kernel<float><<<num_rows, 256, 0, s>>>(x, alpha1, weight1, bias1, (float*)out1, alpha2, weight2, bias2,
-                                                    (float*)out2, width);
+    dyt_pair_kernel<float><<<grid, 256, 0, s>>>(x, alpha1, weight1, bias1, (float*)out1, alpha2, weight2, bias2,
+                                                (float*)out2, width);
   else if (out_dtype == DT_BF16)
-    dyt_pair_kernel<bf16_t><<<num_rows, 256, 0, s>>>(x, alpha1, weight1, bias1, (bf16_t*)out1, alpha2, weight2, bias2,
-                                                     (bf16_t*)out2, width);
+    dyt_pair_kernel<bf16_t><<<grid, 256, 0, s>>>(x, alpha1, weight1, bias1, (bf16_t*)out1, alpha2, weight2, bias2,
+                                                 (bf16_t*)out2, width);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
