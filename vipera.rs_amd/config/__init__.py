@@ -1,5 +1,6 @@
 from .base import KeyReader, LayerSpec, ModelConfig, PartSpec, ScheduleEntry, read_config_json
 from .gilidra import GilidraConfig
+from .lurirax import LuriraxConfig
 from .muzasun import MuzasunConfig
 from .qwen2 import Qwen2Config
 from .zulesun import ZulesunConfig
@@ -15,6 +16,6 @@ from .registry import (
 
 __all__ = [
     "KeyReader", "LayerSpec", "ModelConfig", "PartSpec", "ScheduleEntry", "read_config_json",
-    "GilidraConfig", "MuzasunConfig", "Qwen2Config", "ZulesunConfig", "architecture_names", "architecture_of", "config_from_dict", "load_config",
+    "GilidraConfig", "LuriraxConfig", "MuzasunConfig", "Qwen2Config", "ZulesunConfig", "architecture_names", "architecture_of", "config_from_dict", "load_config",
     "lookup_architecture", "register_architecture", "unregister_architecture",
 ]

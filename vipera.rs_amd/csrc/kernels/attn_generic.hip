@@ -12,7 +12,7 @@
 //
 // Cache layout: K [page, kv_head, slot, head_dim], V transposed [page, kv_head, head_dim, slot];
 // page of position p = table[entry, p / block_size].
-#include "common.h"
+#include "attn_extras.h"
 
 namespace {
 constexpr int THREADS = 256;
@@ -23,7 +23,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     const T* __restrict__ q, long long q_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     T* __restrict__ out, const int* __restrict__ positions, const int* __restrict__ entry_of_token,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, float softcap, const int* __restrict__ skip_single_of) {
+    float scale, int window, float softcap, const int* __restrict__ skip_single_of, AttnExtras ex) {
   // skip_single_of (entry_start, or null): tokens of entries that hold one token are left to the decode kernel
   if (skip_single_of) {
     const int e = entry_of_token[blockIdx.x];
@@ -51,20 +51,26 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
   float acc = 0.f, m = -INFINITY, l = 0.f;
   __syncthreads();
 
-  for (int base = lo; base < hi; base += THREADS) {
-    const int p = base + tid;
+  // the positions that a window keeps beside its own (the first `keep_first`) are walked first: index v of the walk
+  // is position v below `kept`, and position lo + (v - kept) from there on
+  const int kept = min(ex.keep_first, lo);
+  const int hi_v = kept + (hi - lo);
+  for (int base = 0; base < hi_v; base += THREADS) {
+    const int v = base + tid;
+    const int p = v < kept ? v : lo + (v - kept);
     float s = -INFINITY;
     int page = -1;
-    if (p < hi) {
+    if (v < hi_v) {
       page = table[p / block_size];
       const T* k_row = k_cache + (((size_t)page * kv_heads + kvh) * block_size + (p % block_size)) * hd;
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_float<T>(k_row[d]), dot);
       s = capped(dot * scale, softcap);
+      if (ex.rel) s += distance_bias(ex, h, pos - p);
     }
     const float tile_max = block_max(s, red);
     const float m_new = fmaxf(m, tile_max);
-    const float w = (p < hi) ? expf(s - m_new) : 0.f;
+    const float w = (v < hi_v) ? expf(s - m_new) : 0.f;
     const float tile_sum = block_sum(w, red);
     const float rescale = (m == -INFINITY) ? 0.f : expf(m - m_new);
     l = l * rescale + tile_sum;
@@ -74,9 +80,10 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
     __syncthreads();
     if (v_active) {
       acc *= rescale;
-      const int count = min(THREADS, hi - base);
+      const int count = min(THREADS, hi_v - base);
       for (int j = vpart; j < count; j += parts) {
-        const int pj = base + j;
+        const int vj = base + j;
+        const int pj = vj < kept ? vj : lo + (vj - kept);
         const T* v_at = v_cache + (((size_t)page_s[j] * kv_heads + kvh) * hd + vd) * block_size + (pj % block_size);
         acc = fmaf(p_s[j], to_float<T>(*v_at), acc);
       }
@@ -89,7 +96,7 @@ __global__ __launch_bounds__(THREADS) void attn_generic_kernel(
   if (tid < hd) {
     float total = 0.f;
     for (int pidx = 0; pidx < parts; ++pidx) total += part_s[pidx * hd + tid];
-    out[(size_t)t * heads * hd + (size_t)h * hd + tid] = from_float<T>(total / l);
+    out[(size_t)t * heads * hd + (size_t)h * hd + tid] = from_float<T>(total / (l + sink_term(ex, h, m)));
   }
 }
 
@@ -531,11 +538,17 @@ void launch_decode_f32(dim3 grid, hipStream_t s, const float* q, long long q_str
 }
 }  // namespace
 
-extern "C" int vk_attn_generic_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+static bool extras_ok(const AttnExtras& ex, int window) {
+  return ex.rel_far >= 0 && ex.keep_first >= 0 && (ex.keep_first == 0 || window > 0);
+}
+
+extern "C" int vk_attn_generic_ext(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                void* out, int dtype, const int* positions, const int* entry_of_token,
                                const int* block_table, int table_width, int block_size, int num_tokens, int heads,
                                int kv_heads, int hd, float scale, int window, float softcap, const int* skip_single_of,
-                               void* stream) {
+                               const float* sink, const float* rel, int rel_far, int keep_first, void* stream) {
+  const AttnExtras ex{sink, rel, rel_far, keep_first};
+  if (!extras_ok(ex, window)) return VK_BAD_ARGUMENT;
   if (num_tokens <= 0) return 0;
   if (hd <= 0 || hd > MAX_HD) return VK_UNSUPPORTED_SIZE;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || block_size <= 0 || table_width <= 0)
@@ -546,16 +559,26 @@ extern "C" int vk_attn_generic_capped(const void* q, long long q_stride, const v
     attn_generic_kernel<float><<<grid, THREADS, 0, s>>>((const float*)q, q_stride, (const float*)k_cache,
                                                         (const float*)v_cache, (float*)out, positions,
                                                         entry_of_token, block_table, table_width, block_size,
-                                                        heads, kv_heads, hd, scale, window, softcap, skip_single_of);
+                                                        heads, kv_heads, hd, scale, window, softcap, skip_single_of, ex);
   else if (dtype == DT_BF16)
     attn_generic_kernel<bf16_t><<<grid, THREADS, 0, s>>>((const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
                                                          (const bf16_t*)v_cache, (bf16_t*)out, positions,
                                                          entry_of_token, block_table, table_width, block_size,
-                                                         heads, kv_heads, hd, scale, window, softcap, skip_single_of);
+                                                         heads, kv_heads, hd, scale, window, softcap, skip_single_of, ex);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_attn_generic_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                               void* out, int dtype, const int* positions, const int* entry_of_token,
+                               const int* block_table, int table_width, int block_size, int num_tokens, int heads,
+                               int kv_heads, int hd, float scale, int window, float softcap, const int* skip_single_of,
+                               void* stream) {
+  return vk_attn_generic_ext(q, q_stride, k_cache, v_cache, out, dtype, positions, entry_of_token, block_table,
+                             table_width, block_size, num_tokens, heads, kv_heads, hd, scale, window, softcap,
+                             skip_single_of, nullptr, nullptr, 0, 0, stream);
 }
 
 

@@ -19,10 +19,17 @@ constexpr int MOE_TILE = 64;      // places per tile of the 32-bit products; the
 // `groups` > 1: the experts form that many equal groups of neighbours, a group's score is its largest logit, and
 // only experts of the `keep` best groups (the lowest group among equals) can be chosen.  `all_scores` 1: the weights are
 // the chosen experts' shares of the softmax over all E logits, which do not add up to one; 2: the sigmoid of each chosen
-// expert's own logit, not renormalized.
+// expert's own logit, not renormalized; 3: the experts are chosen by sigmoid(logit) + correction[e] (a learned number per
+// expert that steers the choice only) and a chosen expert's weight is weight_scale * sigmoid(logit), not renormalized.
 struct Routing {
   int groups, keep, all_scores;
+  const float* correction = nullptr;
+  float weight_scale = 1.f;
 };
+
+__device__ __forceinline__ float choice_score(const Routing& how, const float* z, int e) {
+  return how.all_scores == 3 ? 1.0f / (1.0f + expf(-z[e])) + (how.correction ? how.correction[e] : 0.f) : z[e];
+}
 
 __device__ __forceinline__ void route_token(const float* __restrict__ logits, int experts, int top, int t, int lane,
                                             int* __restrict__ ids, float* __restrict__ weights,
@@ -35,7 +42,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     const int size = experts / how.groups;
     float score = -INFINITY;
     if (lane < how.groups)
-      for (int e = lane * size; e < (lane + 1) * size; ++e) score = fmaxf(score, z[e]);
+      for (int e = lane * size; e < (lane + 1) * size; ++e) score = fmaxf(score, choice_score(how, z, e));
     unsigned long long kept = 0;
     for (int j = 0; j < how.keep; ++j) {
       float best = (lane < how.groups && !((kept >> lane) & 1ull)) ? score : -INFINITY;
@@ -67,7 +74,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     int arg = NONE;
     for (int e = lane, i = 0; e < experts; e += WAVE, ++i) {
       if ((taken >> i) & 1ull) continue;
-      const float v = z[e];
+      const float v = choice_score(how, z, e);
       if (arg == NONE || v > best) {   // ascending e: an equal later one does not replace
         best = v;
         arg = e;
@@ -83,12 +90,13 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
     }
     if ((arg & (WAVE - 1)) == lane) taken |= 1ull << (arg / WAVE);
     if (j == 0) first = best;
-    const float p = how.all_scores == 2 ? 1.0f / (1.0f + expf(-best)) : how.all_scores ? expf(best - whole_max) : expf(best - first);
+    const float p = how.all_scores == 3 ? how.weight_scale / (1.0f + expf(-z[arg]))
+                    : how.all_scores == 2 ? 1.0f / (1.0f + expf(-best)) : how.all_scores ? expf(best - whole_max) : expf(best - first);
     sum += p;
     if (lane == j) mine = p;
     if (lane == 0) ids[(long long)t * top + j] = arg;
   }
-  if (lane < top) weights[(long long)t * top + lane] = how.all_scores == 2 ? mine : mine / (how.all_scores ? whole_sum : sum);
+  if (lane < top) weights[(long long)t * top + lane] = how.all_scores >= 2 ? mine : mine / (how.all_scores ? whole_sum : sum);
 }
 
 __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int experts, int top,
@@ -376,15 +384,15 @@ extern "C" int vk_moe_tile_rows(int dtype, int width, int ff, long long ldh) {
   return moe_on_matrix_cores(dtype, width, ff, ldh) ? GT_TILE : MOE_TILE;
 }
 
-extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, int num_tokens, int tile_rows, int groups,
-                                    int keep, int all_scores, int* ids, float* weights, int* offsets, int* order,
-                                    int* tiles, int* num_tiles, void* stream) {
+extern "C" int vk_moe_route_steered(const float* logits, int experts, int top, int num_tokens, int tile_rows, int groups,
+                                    int keep, int all_scores, const float* correction, float weight_scale, int* ids,
+                                    float* weights, int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
   if (tile_rows != MOE_TILE && tile_rows != GT_TILE) return VK_BAD_ARGUMENT;
   if (groups < 1 || keep < 1 || keep > groups || experts % groups != 0) return VK_BAD_ARGUMENT;
   if (groups > WAVE) return VK_UNSUPPORTED_SIZE;
   if (keep < groups && (long long)keep * (experts / groups) < top) return VK_BAD_ARGUMENT;
-  if (all_scores < 0 || all_scores > 2) return VK_BAD_ARGUMENT;
-  const Routing how{groups, keep, all_scores};
+  if (all_scores < 0 || all_scores > 3 || (correction && all_scores != 3)) return VK_BAD_ARGUMENT;
+  const Routing how{groups, keep, all_scores, correction, weight_scale};
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
@@ -401,6 +409,14 @@ extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, i
                                                                        offsets, order, tiles, num_tiles, how);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, int num_tokens, int tile_rows, int groups,
+                                    int keep, int all_scores, int* ids, float* weights, int* offsets, int* order,
+                                    int* tiles, int* num_tiles, void* stream) {
+  if (all_scores > 2) return VK_BAD_ARGUMENT;
+  return vk_moe_route_steered(logits, experts, top, num_tokens, tile_rows, groups, keep, all_scores, nullptr, 1.f, ids,
+                              weights, offsets, order, tiles, num_tiles, stream);
 }
 
 extern "C" int vk_moe_route(const float* logits, int experts, int top, int num_tokens, int tile_rows, int* ids,

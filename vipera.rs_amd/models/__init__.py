@@ -4,7 +4,7 @@ from __future__ import annotations
 from .. import parts  # noqa: F401  (registers the built-in parts)
 from ..config.base import ModelConfig
 from ..config.registry import lookup_architecture
-from . import gilidra, muzasun, qwen2, zulesun  # noqa: F401  (register the architectures)
+from . import gilidra, lurirax, muzasun, qwen2, zulesun  # noqa: F401  (register the architectures)
 from .decoder import CacheNeed, DecoderModel, check_model, declare_cache_needs, declare_model
 
 

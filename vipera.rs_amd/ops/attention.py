@@ -8,9 +8,27 @@ workgroup); everything of odd sizes uses the general 32-bit kernel, which serves
 """
 from __future__ import annotations
 
+from dataclasses import dataclass
+from typing import Optional
+
 import torch
 
 from . import kernels
+
+@dataclass
+class AttentionExtras:
+    """What a layer's softmax and mask have beyond scale, window and cap: ``sink`` ([heads] 32-bit: a learned logit per
+    head that joins the denominator and nothing else), ``rel`` ([heads, far + 1] 32-bit: a bias added to the scaled
+    score by the distance between query and key, the last column for every distance from ``far`` on) and
+    ``keep_first`` (with a window: positions below it stay visible).  The attention kernels take them as they take a
+    window."""
+    sink: Optional[torch.Tensor] = None
+    rel: Optional[torch.Tensor] = None
+    keep_first: int = 0
+
+    def any(self) -> bool:
+        return self.sink is not None or self.rel is not None or self.keep_first > 0
+
 
 DECODE_WAVES_WANTED = 512    # enough waves to keep the memory system busy (each keeps a step of loads in flight)
 DECODE_CHUNK_MIN = 128       # below this the merge of the chunks costs more than the waves gain
@@ -112,10 +130,16 @@ def chunks_prompt_tiles(num_tiles: int, heads: int, longest: int, total: int, cu
 
 
 def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, head_dim, scale, window,
-                    softcap: float = 0.0) -> None:
+                    softcap: float = 0.0, extras: Optional[AttentionExtras] = None) -> None:
     """``window`` > 0: a token sees the last that many positions; < 0: the positions of its own block of ``-window``
     consecutive positions, counted from position 0 of its sequence; 0: all before it.  ``softcap`` > 0: a score
-    becomes ``softcap * tanh(score / softcap)`` before the softmax."""
+    becomes ``softcap * tanh(score / softcap)`` before the softmax.  ``extras``: see :class:`AttentionExtras`."""
+    if extras is not None and not extras.any():
+        extras = None
+    if extras is not None:
+        kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
+                             head_dim, scale, window, softcap=softcap, extras=extras)
+        return
     if kernels.attn_bf16_supported(qkv, k_cache, head_dim):
         if batch.num_prefill_tiles:
             cus = kernels.compute_units(qkv.device)

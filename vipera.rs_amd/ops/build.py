@@ -32,7 +32,8 @@ HOST_FLAGS = ["-O2", "-std=c++17", "-shared", "-fPIC", "-Wall"]
 MODULES: Dict[str, tuple] = {
     "elementwise": ("hip", ["kernels/elementwise.hip"], ["kernels/common.h"]),
     "gemm_generic": ("hip", ["kernels/gemm_generic.hip"], ["kernels/common.h"]),
-    "attn_generic": ("hip", ["kernels/attn_generic.hip"], ["kernels/common.h"]),
+    "attn_generic": ("hip", ["kernels/attn_generic.hip"], ["kernels/common.h", "kernels/attn_extras.h"]),
+    "heads": ("hip", ["kernels/heads.hip"], ["kernels/common.h"]),
     "gemm_bf16": ("hip", ["kernels/gemm_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h", "kernels/no_alloc.h"]),
     "sampling": ("hip", ["kernels/sampling.hip"], ["kernels/common.h"]),
     "recurrent": ("hip", ["kernels/recurrent.hip"], ["kernels/common.h"]),

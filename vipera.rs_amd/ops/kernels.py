@@ -254,7 +254,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor],
 def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                  positions: torch.Tensor, entry_of_token: torch.Tensor, block_table: torch.Tensor,
                  heads: int, kv_heads: int, head_dim: int, scale: float, window: int,
-                 skip_single_of: Optional[torch.Tensor] = None, softcap: float = 0.0) -> None:
+                 skip_single_of: Optional[torch.Tensor] = None, softcap: float = 0.0, extras=None) -> None:
     """Causal GQA over the paged cache for every token of the step, in 32-bit arithmetic.  ``window`` > 0: the last
     that many positions; < 0: the positions of the token's own block of ``-window`` consecutive positions (counted
     from position 0); ``softcap`` > 0: scores become ``softcap * tanh(score / softcap)`` (all attention kernels alike).
@@ -277,11 +277,33 @@ def attn_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
     if head_dim > ATTENTION_MAX_HEAD_DIM:
         raise UnsupportedError(f"attention: head_dim {head_dim} is above the kernels' limit of {ATTENTION_MAX_HEAD_DIM}")
-    fn = _fn("attn_generic", "vk_attn_generic_capped",
-             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p])
+    fn = _fn("attn_generic", "vk_attn_generic_ext",
+             [_p, _ll, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p, _p, _i, _i, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _dt(q, "q"), _ptr(positions),
                _ptr(entry_of_token), _ptr(block_table), block_table.shape[1], k_cache.shape[2], num_tokens, heads,
-               kv_heads, head_dim, float(scale), int(window), float(softcap), _ptr(skip_single_of), _stream()), "attn_generic")
+               kv_heads, head_dim, float(scale), int(window), float(softcap), _ptr(skip_single_of),
+               *attn_extras_args(extras, heads, window), _stream()), "attn_generic")
+
+
+def attn_extras_args(extras, heads: int, window: int):
+    """``(sink, rel, rel_far, keep_first)`` as the attention launchers take them; ``extras`` (or None) has the
+    attributes ``sink`` ([heads] 32-bit or None: a learned logit per head that joins the softmax's denominator only),
+    ``rel`` ([heads, rel_far + 1] 32-bit or None: a bias by distance, the last column for every distance from
+    ``rel_far`` on) and ``keep_first`` (positions below it stay visible to a windowed layer)."""
+    if extras is None:
+        return _p(0), _p(0), 0, 0
+    sink, rel, keep_first = extras.sink, extras.rel, int(extras.keep_first or 0)
+    _dev(sink, rel)
+    rel_far = 0
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and sink.is_contiguous() and sink.numel() == heads,
+              "attention: one 32-bit sink logit per query head")
+    if rel is not None:
+        _need(rel.dtype == torch.float32 and rel.is_contiguous() and rel.dim() == 2 and rel.shape[0] == heads
+              and rel.shape[1] >= 1, "attention: the bias by distance is [heads, distances] in 32-bit")
+        rel_far = rel.shape[1] - 1
+    _need(keep_first >= 0 and (keep_first == 0 or window > 0), "attention: kept first positions need a window")
+    return _ptr(sink), _ptr(rel), rel_far, keep_first
 
 
 ATTN_DECODE_F32_CHUNK = 256   # positions of one workgroup of attn_decode_f32 (the kernel's DEC_CHUNK)
@@ -1234,13 +1256,15 @@ def moe_max_tiles(pairs: int, experts: int, tile_rows: int = 64) -> int:
 
 def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor, offsets: torch.Tensor,
               order: torch.Tensor, tiles: torch.Tensor, num_tiles: torch.Tensor, tile_rows: int = 64,
-              groups: int = 1, keep: int = 1, all_scores=False) -> None:
+              groups: int = 1, keep: int = 1, all_scores=False, correction: Optional[torch.Tensor] = None,
+              weight_scale: float = 1.0) -> None:
     """Each token's ``top`` largest router logits (lowest id first among equals) with the softmax over those, and the
     (token, choice) pairs grouped by expert: ``offsets [E + 1]``, ``order [T * top]``, ``tiles [max, 2]``.
     ``groups`` > 1: the experts form that many equal groups of neighbours and only those of the ``keep`` groups with
     the largest logits can be chosen.  ``all_scores``: the weights are the chosen experts' shares of the softmax over
     all experts (they do not add up to one); ``all_scores="sigmoid"``: the weight of a chosen expert is the sigmoid of its
-    own logit, not renormalized."""
+    own logit, not renormalized; ``all_scores="steered"``: the experts are chosen by ``sigmoid(logit) + correction[e]``
+    (``correction`` [experts] 32-bit or None) and a chosen expert's weight is ``weight_scale * sigmoid(logit)``."""
     _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
     tokens, experts = logits.shape
     _f32(logits, "moe_route: logits")
@@ -1252,9 +1276,15 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
           and num_tiles.numel() == 1 and tile_rows in (64, 128), "moe_route: output sizes")
     _need(1 <= keep <= groups <= 64 and experts % groups == 0 and (keep == groups or keep * (experts // groups) >= top),
           f"moe_route: {keep} of {groups} groups of {experts} experts for top {top}")
-    fn = _fn("moe", "vk_moe_route_grouped", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p])
-    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), 2 if all_scores == "sigmoid" else 1 if all_scores else 0, _ptr(ids),
-               _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles), _ptr(num_tiles), _stream()), "moe_route")
+    mode = {"sigmoid": 2, "steered": 3}.get(all_scores, 1 if all_scores else 0)
+    if correction is not None:
+        _dev(correction)
+        _need(mode == 3 and correction.dtype == torch.float32 and correction.is_contiguous()
+              and correction.numel() == experts, "moe_route: one 32-bit correction per expert, with steered scores")
+    fn = _fn("moe", "vk_moe_route_steered", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p, _p, _p, _p, _p, _p, _p])
+    _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), mode, _ptr(correction),
+               float(weight_scale), _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles), _ptr(num_tiles),
+               _stream()), "moe_route")
 
 
 def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
@@ -1558,3 +1588,89 @@ def scan_prepare(dt: torch.Tensor, dt_bias: torch.Tensor, z: torch.Tensor, gate:
     fn = _fn("scan", "vk_scan_prepare", [_p, _ll, _p, _p, _ll, _p, _i, _i, _p])
     _status(fn(_ptr(dt), dt.stride(0), _ptr(dt_bias), _ptr(z), z.stride(0), _ptr(gate), tokens, channels, _stream()),
             "scan_prepare")
+
+
+# ----------------------------------------------------------------------------------------------
+_GATE_ACTS = {"none": 0, "silu": 2, "sigmoid": 4}
+
+
+def head_prepare(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], norm: bool,
+                 norm_first: bool, eps: float, positions: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
+                 rot_dims: int, heads: int, kv_heads: int, maps: int, dim: int, vdim: int, width: int,
+                 qkv: torch.Tensor) -> None:
+    """The 32-bit sums ``proj`` = ``[q | k | v | ...]`` of a step's tokens laid out head by head at one padded
+    ``width`` in ``qkv``: q and k heads rotated by position (the first ``rot_dims`` numbers, half-split pairs) and, with
+    ``norm``, divided by their root mean square and multiplied by a weight of ``dim`` numbers (None: no weight), before
+    the rotation (``norm_first``) or behind it.  ``maps`` > 1: that many attention maps per head; a query head's maps
+    become query heads of their own, each in its own columns of the padded width, and a key head's maps stay side by
+    side in one key head, so every map meets its own keys and all maps of a head read the same values."""
+    _dev(proj, q_weight, k_weight, positions, inv_freq, qkv)
+    tokens = proj.shape[0]
+    need = (heads + kv_heads) * maps * dim + kv_heads * vdim
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= need,
+          "head_prepare: proj must be 32-bit [tokens, >= q + k + v columns]")
+    _need(qkv.shape == (tokens, (heads * maps + 2 * kv_heads) * width) and qkv.is_contiguous(), "head_prepare: qkv shape")
+    _need(width >= maps * dim and width >= vdim and dim <= 256, "head_prepare: the padded width holds every head")
+    for weight in (q_weight, k_weight):
+        if weight is not None:
+            _need(weight.dtype == torch.float32 and weight.numel() == dim and weight.is_contiguous(), "head_prepare: weights")
+    if rot_dims:
+        _need(rot_dims % 2 == 0 and rot_dims <= dim and positions is not None and positions.dtype == torch.int32
+              and positions.numel() >= tokens and inv_freq is not None and inv_freq.dtype == torch.float32
+              and inv_freq.numel() == rot_dims // 2, "head_prepare: rotation operands")
+    fn = _fn("heads", "vk_head_prepare", [_p, _ll, _p, _p, _i, _i, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p])
+    _status(fn(_ptr(proj), proj.stride(0), _ptr(q_weight), _ptr(k_weight), 1 if norm else 0, 1 if norm_first else 0,
+               float(eps), _ptr(positions), _ptr(inv_freq), int(rot_dims), tokens, heads, kv_heads, maps, dim, vdim,
+               width, _ptr(qkv), _dt(qkv, "qkv"), _stream()), "head_prepare")
+
+
+def head_finish(attn: torch.Tensor, out: torch.Tensor, heads: int, vdim: int, width: int, maps: int = 1,
+                subtract: float = 0.0, unit_norm: bool = False, eps: float = 0.0, factor: float = 1.0,
+                gate: Optional[torch.Tensor] = None, gate_kind: str = "none", gate_per_head: bool = False) -> None:
+    """The attention kernels' output (``heads * maps`` heads of padded ``width``) becomes the output product's input
+    ``out [tokens, heads * vdim]``: with two maps ``a_1 - subtract * a_2``; with ``unit_norm`` divided by the head's
+    root mean square; times ``factor``; times ``gate_kind(gate)``, one 32-bit number per head (``gate_per_head``,
+    ``gate [tokens, >= heads]``) or per number (``gate [tokens, >= heads * vdim]``)."""
+    _dev(attn, out, gate)
+    tokens = attn.shape[0]
+    _need(attn.shape == (tokens, heads * maps * width) and attn.is_contiguous() and maps in (1, 2), "head_finish: attn shape")
+    _need(out.shape == (tokens, heads * vdim) and out.is_contiguous() and out.dtype == attn.dtype, "head_finish: out shape")
+    _need(vdim <= width and vdim <= 256, "head_finish: widths")
+    _need(gate_kind in _GATE_ACTS, f"head_finish: gate {gate_kind!r}")
+    ldg = 0
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == tokens and gate.stride(1) == 1
+              and gate.shape[1] >= (heads if gate_per_head else heads * vdim), "head_finish: gate shape")
+        ldg = gate.stride(0)
+    fn = _fn("heads", "vk_head_finish", [_p, _i, _i, _f, _i, _f, _f, _p, _ll, _i, _i, _i, _i, _i, _i, _p, _p])
+    _status(fn(_ptr(attn), _dt(attn, "attn"), maps, float(subtract), 1 if unit_norm else 0, float(eps), float(factor),
+               _ptr(gate), ldg, 1 if gate_per_head else 0, _GATE_ACTS[gate_kind], tokens, heads, vdim, width, _ptr(out),
+               _stream()), "head_finish")
+
+
+def rotate_scale(x: torch.Tensor, positions: torch.Tensor, inv_freq: Optional[torch.Tensor], rot_dims: int, heads: int,
+                 dim: int, factor: float = 1.0) -> None:
+    """``heads`` heads of ``dim`` 32-bit numbers from column 0 of ``x`` (rows may be strided) rotated in place by their
+    token's position (the first ``rot_dims`` numbers, half-split pairs) and multiplied by ``factor``."""
+    _dev(x, positions, inv_freq)
+    tokens = x.shape[0]
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1 and x.shape[1] >= heads * dim, "rotate_scale: x")
+    _need(rot_dims % 2 == 0 and 0 <= rot_dims <= dim, "rotate_scale: rot_dims")
+    if rot_dims:
+        _need(positions.dtype == torch.int32 and positions.numel() >= tokens and inv_freq is not None
+              and inv_freq.dtype == torch.float32 and inv_freq.numel() == rot_dims // 2, "rotate_scale: rotation operands")
+    fn = _fn("heads", "vk_rotate_scale", [_p, _ll, _p, _p, _i, _i, _i, _i, _f, _p])
+    _status(fn(_ptr(x), x.stride(0), _ptr(positions), _ptr(inv_freq), int(rot_dims), tokens, heads, dim, float(factor),
+               _stream()), "rotate_scale")
+
+
+def row_gate_add(y: torch.Tensor, gate: torch.Tensor, gate_kind: str, out: torch.Tensor, accumulate: bool = True) -> None:
+    """``out[r, :] (+)= gate_kind(gate[r]) * y[r, :]``: 32-bit rows gated by one number each (``gate [rows, >= 1]``)."""
+    _dev(y, gate, out)
+    _need(y.dtype == torch.float32 and out.dtype == torch.float32 and y.shape == out.shape and y.dim() == 2
+          and y.is_contiguous() and out.is_contiguous(), "row_gate_add: two contiguous 32-bit matrices of one shape")
+    _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == y.shape[0], "row_gate_add: gate")
+    _need(gate_kind in _GATE_ACTS, f"row_gate_add: gate {gate_kind!r}")
+    fn = _fn("heads", "vk_row_gate_add", [_p, _p, _ll, _i, _p, _i, _i, _i, _p])
+    _status(fn(_ptr(y), _ptr(gate), gate.stride(0), _GATE_ACTS[gate_kind], _ptr(out), y.shape[0], y.shape[1],
+               1 if accumulate else 0, _stream()), "row_gate_add")

@@ -30,6 +30,7 @@ LAUNCHERS = (
     "latent_kv_write", "latent_q_rotate", "head_linear", "moe_route", "moe_experts",
     "rmsnorm_add", "axpby", "activation", "whole_norm_pack", "head_unpack_gate", "decay_rule", "gated_norm",
     "causal_conv", "selective_scan", "scan_prepare", "head_norm_pack", "channel_decay", "memory_rule", "dyt_pair",
+    "head_prepare", "head_finish", "rotate_scale", "row_gate_add",
 )
 
 

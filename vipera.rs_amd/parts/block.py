@@ -7,6 +7,8 @@ reference (crates/vipera-backend-cpu/src/model.rs:3-4, 975-1198).
 ``sandwich_norm``: a norm before and behind each sublayer, ``x += norm_1b(mixer(norm_1(x))); x += norm_2b(ffn(norm_2(x)))``,
 and optionally a part that adds to the stream after both (``extras["after"]``, of the feed-forward family; it reads the
 32-bit stream itself).  The norms behind the sublayers are ``extras["mixer_post_norm"]`` and ``extras["ffn_post_norm"]``.
+``postnorm``: a norm behind each sublayer only, ``x += norm_1(mixer(x)); x += norm_2(ffn(x))``; the sublayers read the
+stream itself (``LayerSpec.mixer_norm`` and ``ffn_norm`` are the two norms behind).
 """
 from __future__ import annotations
 
@@ -223,6 +225,87 @@ class SandwichBlock(Block):
             after.forward(stream if feeds_after else None, batch, x)
 
 
+class PostNormBlock(Block):
+    """``x += norm_1(mixer(x)); x += norm_2(ffn(x))``: nothing stands in front of a sublayer, which reads the 32-bit
+    stream in the run's dtype; its output goes into a 32-bit buffer of its own and is normed there and added to the
+    stream by one kernel, which also hands the new stream on in the run's dtype for the sublayer that follows (this
+    layer's feed-forward, or the next layer's mixer through ``batch.shared``)."""
+
+    STREAM_KEY = "postnorm.stream"     # (the stream tensor, its rows in the run's dtype) as the layer before left them
+
+    def __init__(self, spec: LayerSpec, runtime):
+        super().__init__(spec, runtime)
+        self.mixer_post = part_class("norm", spec.mixer_norm.kind)(spec.mixer_norm, spec.prefix, runtime)
+        self.mixer = part_class("mixer", spec.mixer.kind)(spec.mixer, spec.prefix, runtime)
+        self.position = part_class("position", spec.position.kind)(spec.position, spec.prefix, runtime)
+        self.has_ffn = spec.ffn.kind != "none"
+        self.ffn = self.ffn_post = None
+        if self.has_ffn:
+            self.ffn = part_class("ffn", spec.ffn.kind)(spec.ffn, spec.prefix, runtime)
+            self.ffn_post = part_class("norm", spec.ffn_norm.kind)(spec.ffn_norm, spec.prefix, runtime)
+
+    @classmethod
+    def _families(cls, spec: LayerSpec):
+        parts = [("norm", spec.mixer_norm), ("mixer", spec.mixer), ("position", spec.position)]
+        if spec.ffn.kind != "none":
+            parts += [("ffn", spec.ffn), ("norm", spec.ffn_norm)]
+        return parts
+
+    @classmethod
+    def declare(cls, spec: LayerSpec) -> List[TensorSpec]:
+        out: List[TensorSpec] = []
+        for family, part in cls._families(spec):
+            out += part_class(family, part.kind).declare(part, spec.prefix)
+        if spec.ffn.kind == "none":
+            # a layer without a feed-forward does not read the norm behind it; a folder may hold it all the same
+            out += [TensorSpec(t.name, t.shape, t.role, t.init, t.std, True)
+                    for t in part_class("norm", spec.ffn_norm.kind).declare(spec.ffn_norm, spec.prefix)]
+        return out
+
+    @classmethod
+    def check_supported(cls, spec: LayerSpec, dtype) -> None:
+        for family, part in cls._families(spec):
+            part_class(family, part.kind).check_supported(part, dtype)
+
+    def load(self, tensors) -> None:
+        for part in (self.mixer_post, self.mixer, self.position, self.ffn, self.ffn_post):
+            if part is not None:
+                part.load(tensors)
+
+    def _as_input(self, x, batch):
+        import torch
+        from ..ops import kernels
+        left = batch.shared.pop(self.STREAM_KEY, None)
+        if left is not None and left[0] is x:
+            return left[1]
+        if self.runtime.dtype == torch.float32:
+            return x
+        h = self.runtime.empty(tuple(x.shape))
+        kernels.activation(x, "none", h)            # a change of type
+        return h
+
+    def _sublayer(self, run, part, x):
+        import torch
+        if part.can_overwrite:
+            y = torch.empty_like(x)
+            run(y, {"accumulate": False})
+        else:
+            y = torch.zeros_like(x)
+            run(y, {})
+        return y
+
+    def forward(self, x, batch, cache, state, reads_only: bool = False) -> None:
+        h = self._as_input(x, batch)
+        y = self._sublayer(lambda out, kw: self.mixer.forward(h, batch, cache, state, self.position, out, reads_only, **kw),
+                           self.mixer, x)
+        h = self.mixer_post.add_into(y, x, as_input=True)
+        if self.has_ffn:
+            y = self._sublayer(lambda out, kw: self.ffn.forward(h, batch, out, **kw), self.ffn, x)
+            h = self.ffn_post.add_into(y, x, as_input=True)
+        batch.shared[self.STREAM_KEY] = (x, h)
+
+
 register_block("prenorm", PreNormBlock)
+register_block("postnorm", PostNormBlock)
 register_block("sandwich_norm", SandwichBlock)
 register_block("parallel", ParallelBlock)

@@ -34,8 +34,9 @@ class GatedMLP(FeedForward):
         super().__init__(spec, prefix, runtime)
         self.hidden = int(spec.params["hidden"])
         self.inter = int(spec.params["intermediate"])
-        if spec.params.get("activation", "silu") != "silu":
-            raise UnsupportedError(f"activation {spec.params.get('activation')!r} is not implemented; only \"silu\"")
+        self.activation = spec.params.get("activation", "silu")
+        if self.activation not in ("silu", "gelu_tanh"):
+            raise UnsupportedError(f"activation {self.activation!r} is not implemented; \"silu\" or \"gelu_tanh\"")
         self.w_gate_up = self.w_down = None
         self.interleaved = False
 
@@ -54,7 +55,8 @@ class GatedMLP(FeedForward):
         gate, up = tensors[gate_name], tensors[up_name]
         # all-bfloat16 weights of a width the kernels can pair are interleaved, so that the product's
         # epilogue can apply the gate; anything else stays [gate; up]
-        self.interleaved = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0)
+        self.interleaved = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0
+                            and self.activation == "silu")
         self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
         self.w_down = tensors[down_name]
 
@@ -73,10 +75,17 @@ class GatedMLP(FeedForward):
 
     fills_handoff = True
 
-    def forward(self, h, batch, residual, handoff=None, outgoing=None) -> None:
+    can_overwrite = True
+
+    def forward(self, h, batch, residual, handoff=None, outgoing=None, accumulate: bool = True) -> None:
         tokens = residual.shape[0]
         act = self.runtime.empty((tokens, self.inter))
-        if handoff is not None and self._dividing_plan(tokens) == 0:
+        if self.activation != "silu":
+            # another gate than silu: the product's 32-bit sums, then act(gate) * up in one pass
+            both = torch.empty((tokens, 2 * self.inter), dtype=torch.float32, device=residual.device)
+            linear(h, self.w_gate_up, None, both)
+            kernels.activation(both[:, :self.inter], self.activation, act, mul=both[:, self.inter:])
+        elif handoff is not None and self._dividing_plan(tokens) == 0:
             kernels.gemm_bf16_gated_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups, handoff.eps)
         elif handoff is not None:
             kernels.gemm_bf16_gated_tile_scaled(handoff.scaled, self.w_gate_up, act, handoff.sumsq, handoff.groups,
@@ -87,7 +96,7 @@ class GatedMLP(FeedForward):
             # the down product also prepares the next layer's first norm where its kernel can
             outgoing.groups = linear_follow(act, self.w_down, None, residual, outgoing.gain, outgoing.scaled, outgoing.sumsq)
         else:
-            linear(act, self.w_down, None, residual, accumulate=True)
+            linear(act, self.w_down, None, residual, accumulate=accumulate)
 
 
 class NoFeedForward(FeedForward):

@@ -8,9 +8,12 @@ a ``limit`` nothing is clamped and ``y = g * sigmoid(alpha * g) * u`` (``alpha``
 ``keep``: the experts form that many equal groups of neighbours, a group's score is its largest logit, and only experts
 of the ``keep`` best groups can be chosen.  ``scores: "all"``: the weights are the chosen experts' shares of the softmax
 over all experts, not renormalized; ``scores: "sigmoid"``: a chosen expert's weight is the sigmoid of its own logit, not
-renormalized.  ``weigh: "input"``: the weight multiplies what the expert reads instead of what it returns, so the layer
+renormalized; ``scores: "steered"``: the experts are chosen by ``sigmoid(z) + correction`` (a learned number per
+expert, tensor ``<name>.correction``, that steers the choice and nothing else) and a chosen expert's weight is
+``weight_scale * sigmoid(z)``, not renormalized.  ``weigh: "input"``: the weight multiplies what the expert reads instead of what it returns, so the layer
 adds the sum of ``expert(w h)``.  ``shared``: a gated feed-forward of that width (``silu(Wg h) * (Wu h)`` through
-``Wd``, tensors ``<name>.shared.gate | up | down``) that every token runs beside its experts.
+``Wd``, tensors ``<name>.shared.gate | up | down``) that every token runs beside its experts; with ``shared_gate``
+("sigmoid") its output is multiplied by ``sigmoid(Wsg h)``, one number per token (tensor ``<name>.shared.sg``).
 
 The step's (token, choice) pairs are grouped by expert on the device, so nothing about the routing reaches the
 host and a step of single tokens can be captured; see ``csrc/kernels/moe.hip``.
@@ -25,7 +28,7 @@ from ..config.base import PartSpec
 from ..errors import InvalidArgumentError, UnsupportedError
 from ..ops import kernels
 from ..ops.linear import linear
-from ..weights.checkpoint import MATRIX, TensorSpec
+from ..weights.checkpoint import MATRIX, VECTOR, TensorSpec
 from .base import FeedForward, register_ffn
 
 
@@ -43,7 +46,10 @@ class MixtureOfExperts(FeedForward):
         self.limit = float(p["limit"]) if p.get("limit") is not None else float("inf")
         self.alpha = float(p.get("alpha", 1.702))
         self.groups, self.keep = int(p.get("groups") or 1), int(p.get("keep") or p.get("groups") or 1)
-        self.all_scores = {"chosen": False, "all": True, "sigmoid": "sigmoid"}[p.get("scores", "chosen")]
+        self.all_scores = {"chosen": False, "all": True, "sigmoid": "sigmoid", "steered": "steered"}[p.get("scores", "chosen")]
+        self.weight_scale = float(p.get("weight_scale", 1.0))
+        self.shared_gate = p.get("shared_gate")
+        self.correction = self.w_shared_gate = None
         self.weigh_input = p.get("weigh", "output") == "input"
         self.shared = None
         if p.get("shared"):
@@ -70,9 +76,13 @@ class MixtureOfExperts(FeedForward):
                       TensorSpec(f"{base}e{e}.up", (inter, hidden), MATRIX),
                       TensorSpec(f"{base}e{e}.down", (hidden, inter), MATRIX)]
         specs.append(TensorSpec(base + "router", (int(p["experts"]), hidden), MATRIX))
+        if p.get("scores") == "steered":
+            specs.append(TensorSpec(base + "correction", (int(p["experts"]),), VECTOR, std=0.1))
         if p.get("shared"):
             from .mlp import GatedMLP
             specs += GatedMLP.declare(cls._shared_spec(p), prefix)
+            if p.get("shared_gate"):
+                specs.append(TensorSpec(base + "shared.sg", (1, hidden), MATRIX))
         return specs
 
     @classmethod
@@ -88,9 +98,11 @@ class MixtureOfExperts(FeedForward):
         if groups < 1 or experts % groups or not 1 <= keep <= groups or (keep < groups and keep * (experts // groups) < top):
             raise InvalidArgumentError(f"mixture of experts: {keep} of {groups} groups of {experts} experts cannot "
                                        f"give a token its {top}")
-        if spec.params.get("scores", "chosen") not in ("chosen", "all", "sigmoid"):
-            raise UnsupportedError(f"mixture of experts: scores {spec.params.get('scores')!r}; \"chosen\", \"all\" or "
-                                   "\"sigmoid\"")
+        if spec.params.get("scores", "chosen") not in ("chosen", "all", "sigmoid", "steered"):
+            raise UnsupportedError(f"mixture of experts: scores {spec.params.get('scores')!r}; \"chosen\", \"all\", "
+                                   "\"sigmoid\" or \"steered\"")
+        if spec.params.get("shared_gate") not in (None, "sigmoid"):
+            raise UnsupportedError(f"mixture of experts: shared_gate {spec.params.get('shared_gate')!r}; \"sigmoid\" or none")
         if spec.params.get("weigh", "output") not in ("output", "input"):
             raise UnsupportedError(f"mixture of experts: weigh {spec.params.get('weigh')!r}; \"output\" or \"input\"")
 
@@ -100,8 +112,12 @@ class MixtureOfExperts(FeedForward):
         stack = lambda kind: torch.stack([tensors[f"{base}e{e}.{kind}"].to(dtype) for e in range(self.experts)]).contiguous()
         self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
         self.w_router = tensors[base + "router"]
+        if self.all_scores == "steered":
+            self.correction = tensors[base + "correction"]
         if self.shared is not None:
             self.shared.load(tensors)
+            if self.shared_gate:
+                self.w_shared_gate = tensors[base + "shared.sg"]
 
     can_overwrite = True
 
@@ -120,13 +136,21 @@ class MixtureOfExperts(FeedForward):
         tiles = ints[2 * pairs + self.experts + 2:]
         weights = torch.empty(pairs, dtype=torch.float32, device=device)
         kernels.moe_route(logits, self.top, ids, weights, offsets, order, tiles, num_tiles, tile_rows,
-                          groups=self.groups, keep=self.keep, all_scores=self.all_scores)
+                          groups=self.groups, keep=self.keep, all_scores=self.all_scores, correction=self.correction,
+                          weight_scale=self.weight_scale)
         act = self.runtime.empty((pairs, self.inter))
         pair_out = torch.empty((pairs, self.hidden), dtype=torch.float32, device=device)
         kernels.moe_experts(h, self.w_gate, self.w_up, self.w_down, offsets, order, tiles, num_tiles, weights,
                             self.top, self.limit, self.alpha, act, pair_out, residual, accumulate, self.weigh_input)
-        if self.shared is not None:
+        if self.shared is not None and self.w_shared_gate is None:
             self.shared.forward(h, batch, residual)
+        elif self.shared is not None:
+            # the shared expert into a buffer of its own, which joins the others' sum times the token's gate
+            own = torch.zeros_like(residual)
+            self.shared.forward(h, batch, own)
+            gate = torch.empty((tokens, 1), dtype=torch.float32, device=device)
+            linear(h, self.w_shared_gate, None, gate)
+            kernels.row_gate_add(own, gate, self.shared_gate, residual)
 
 
 register_ffn("moe", MixtureOfExperts)

@@ -24,7 +24,9 @@ goes through ``Wo``.
 ``decay_attention``: linear attention whose heads forget at a fixed rate each.  ``q = act(Wq h)``, ``k = act(Wk h)``
 (``heads x dim``), ``v = act(Wv h)`` (``heads x vdim``); per head ``S <- decay_h S + k v^T; o = S^T q``; the heads'
 outputs are normed together (one RMS norm over ``heads * vdim`` numbers), gated by ``sigmoid(Wg h)`` and go through
-``Wo``.
+``Wo``.  Options: ``rotary`` (q and k rotated by position before they enter the recurrence, as an attention layer's
+are), ``k_scale`` (k multiplied by it behind the rotation), ``norm: "head"`` (every head's output divided by its own
+root mean square, no weight: retention).
 
 ``selective_scan``: Mamba.  ``W_in h = [x | z]``; x passes a short causal convolution per channel with a bias, and
 silu; ``W_x x = [dt | B | C]``; ``step = softplus(W_dt dt + dt_bias)``; per channel c and state n
@@ -237,7 +239,9 @@ class MatrixMemory(Mixer):
         bias[-2 * self.heads:-self.heads] = tensors[base + "i.b"].float()
         bias[-self.heads:] = tensors[base + "f.b"].float()
         self.b_in = bias
-        self.w_o, self.norm = tensors[base + "o"], tensors[base + "norm"]
+        self.w_o = tensors[base + "o"]
+        if self.norm_kind == "whole":
+            self.norm = tensors[base + "norm"]
 
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
         tokens, entries = residual.shape[0], batch.num_entries
@@ -343,7 +347,9 @@ class Wkv(Mixer):
 class DecayAttention(Mixer):
     """``params``: ``hidden``, ``heads``, ``dim``, ``vdim``, ``decay`` (one number per head), ``eps`` (of the read-out's
     norm), ``activation`` ("silu" or "none", of q, k and v), ``gate`` ("sigmoid", "silu" or "none"), ``name``; tensors
-    ``<name>.q | k | v | g | o | norm``."""
+    ``<name>.q | k | v | g | o | norm``.  Optional: ``rotary`` (``{"dims", "base"}``: the first ``dims`` numbers of every
+    q and k head rotate by position in half-split pairs, in 32-bit), ``k_scale`` (1 unless given), ``norm`` ("whole":
+    one norm over all heads with the weight ``norm``; "head": each head over its own root mean square, no tensor)."""
 
     can_overwrite = True
 
@@ -361,16 +367,30 @@ class DecayAttention(Mixer):
         self.decay = torch.tensor(rates, dtype=torch.float32, device=runtime.device)
         self.qk, self.vw = self.heads * self.dim, self.heads * self.vdim
         self.w_in = self.w_o = self.norm = None
+        self.k_scale = float(p.get("k_scale") or 1.0)
+        self.norm_kind = p.get("norm", "whole")
+        rotary = p.get("rotary") or {}
+        self.rot_dims = int(rotary.get("dims") or 0)
+        self.inv_freq = None
+        if self.rot_dims:
+            from .rotary import neox_inverse_frequencies
+            if self.rot_dims % 2 or self.rot_dims > self.dim:
+                raise InvalidArgumentError(f"decay_attention: {self.rot_dims} rotated numbers of a head of {self.dim}")
+            self.inv_freq = torch.from_numpy(neox_inverse_frequencies(self.rot_dims, float(rotary["base"]))).to(runtime.device)
+        if self.norm_kind == "head":
+            self.norm = torch.ones(self.vdim, dtype=torch.float32, device=runtime.device)
 
     @classmethod
     def declare(cls, spec: PartSpec, prefix: str) -> List[TensorSpec]:
         p = spec.params
         base = f"{prefix}{p['name']}."
         hidden, qk, vw = int(p["hidden"]), int(p["heads"]) * int(p["dim"]), int(p["heads"]) * int(p["vdim"])
-        return [TensorSpec(base + "q", (qk, hidden), MATRIX), TensorSpec(base + "k", (qk, hidden), MATRIX),
-                TensorSpec(base + "v", (vw, hidden), MATRIX), TensorSpec(base + "g", (vw, hidden), MATRIX),
-                TensorSpec(base + "o", (hidden, vw), MATRIX),
-                TensorSpec(base + "norm", (vw,), VECTOR, "one_plus_normal")]
+        specs = [TensorSpec(base + "q", (qk, hidden), MATRIX), TensorSpec(base + "k", (qk, hidden), MATRIX),
+                 TensorSpec(base + "v", (vw, hidden), MATRIX), TensorSpec(base + "g", (vw, hidden), MATRIX),
+                 TensorSpec(base + "o", (hidden, vw), MATRIX)]
+        if p.get("norm", "whole") == "whole":
+            specs.append(TensorSpec(base + "norm", (vw,), VECTOR, "one_plus_normal"))
+        return specs
 
     @classmethod
     def declare_cache(cls, spec: PartSpec):
@@ -382,11 +402,15 @@ class DecayAttention(Mixer):
         if int(spec.params["dim"]) > kernels.DECAY_RULE_MAX_KEY_DIM:
             raise UnsupportedError(f"decay_attention: a key width of {spec.params['dim']} is above the kernel's limit of "
                                    f"{kernels.DECAY_RULE_MAX_KEY_DIM}")
+        if spec.params.get("norm", "whole") not in ("whole", "head"):
+            raise UnsupportedError(f"decay_attention: norm {spec.params.get('norm')!r}; \"whole\" or \"head\"")
 
     def load(self, tensors: Dict[str, torch.Tensor]) -> None:
         base = f"{self.prefix}{self.spec.params['name']}."
         self.w_in = _cat([tensors[base + n] for n in ("q", "k", "v", "g")])     # one product for all that reads h
-        self.w_o, self.norm = tensors[base + "o"], tensors[base + "norm"]
+        self.w_o = tensors[base + "o"]
+        if self.norm_kind == "whole":
+            self.norm = tensors[base + "norm"]
 
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
         tokens, entries = residual.shape[0], batch.num_entries
@@ -397,6 +421,12 @@ class DecayAttention(Mixer):
         v, g = proj[:, 2 * self.qk:2 * self.qk + self.vw], proj[:, 2 * self.qk + self.vw:]
         o = torch.empty((tokens, self.vw), **f32)
         inside = self.activation == "silu"
+        if self.rot_dims or self.k_scale != 1.0:
+            if inside:
+                raise UnsupportedError("decay_attention: a rotation behind an activation of q and k is not implemented")
+            if self.rot_dims:
+                kernels.rotate_scale(q, batch.positions, self.inv_freq, self.rot_dims, self.heads, self.dim)
+            kernels.rotate_scale(k, batch.positions, self.inv_freq, self.rot_dims, self.heads, self.dim, self.k_scale)
         if inside and not batch.all_single:
             # every workgroup of value channels would take the activation of a token's q and k again, token behind
             # token: a prompt's portion takes it once, ahead of the recurrence; a step of single tokens saves the launch
@@ -408,7 +438,12 @@ class DecayAttention(Mixer):
         kernels.decay_rule(q, k, v, inside, self.decay, state, batch.entry_start,
                            batch.entry_first_pos, batch.slots, self.heads, self.dim, self.vdim, o, entries)
         gated = self.runtime.empty((tokens, self.vw))
-        kernels.gated_norm(o, self.norm, g, self.gate, self.eps, gated)
+        if self.norm_kind == "head":
+            if self.gate == "none":
+                raise UnsupportedError("decay_attention: a norm per head without a gate is not implemented")
+            kernels.head_norm_gate(o, self.norm, g, self.gate, self.eps, self.heads, self.vdim, gated)
+        else:
+            kernels.gated_norm(o, self.norm, g, self.gate, self.eps, gated)
         linear(gated, self.w_o, None, residual, accumulate=accumulate)
 
 

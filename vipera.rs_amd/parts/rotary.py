@@ -28,6 +28,17 @@ def neox_inverse_frequencies(rotary_dim: int, base: float) -> np.ndarray:
     return (np.float32(1.0) / np.power(np.float32(base), exponent, dtype=np.float32)).astype(np.float32)
 
 
+def stretch_long_waves(table: np.ndarray, factor: float, low: float, high: float, original: float) -> np.ndarray:
+    """Frequencies scaled by wavelength, as Llama 3.1 stretches its context: with ``l = 2 pi / f``, a frequency stays
+    where ``l < original / high``, is divided by ``factor`` where ``l > original / low``, and in between is blended,
+    ``(1 - s) f / factor + s f`` with ``s = (original / l - low) / (high - low)``."""
+    f = table.astype(np.float64)
+    wave = 2.0 * np.pi / f
+    share = (original / wave - low) / (high - low)
+    out = np.where(wave < original / high, f, np.where(wave > original / low, f / factor, (1.0 - share) * f / factor + share * f))
+    return out.astype(np.float32)
+
+
 class RotaryNeox(PositionEncoding):
     def __init__(self, spec: PartSpec, prefix: str, runtime):
         super().__init__(spec, prefix, runtime)
@@ -42,6 +53,11 @@ class RotaryNeox(PositionEncoding):
         table = neox_inverse_frequencies(self.rotary_dim, self.base)
         if self.scaling_factor != 1.0:
             table = (table / np.float32(self.scaling_factor)).astype(np.float32)
+        # ``long_waves``: {"factor", "low", "high", "original"}, see stretch_long_waves
+        self.long_waves = spec.params.get("long_waves")
+        if self.long_waves and self.rotary_dim:
+            w = self.long_waves
+            table = stretch_long_waves(table, float(w["factor"]), float(w["low"]), float(w["high"]), float(w["original"]))
         self.inv_freq = torch.from_numpy(table).to(runtime.device)
 
     def fused_rotary(self):
@@ -52,7 +68,8 @@ class RotaryNeox(PositionEncoding):
         # again; a few decoded tokens are cheaper without the extra launch
         if batch.num_tokens < ANGLE_TABLE_MIN_TOKENS or not self.rotary_dim:
             return None
-        key = ("rope_angles", self.base, self.rotary_dim, self.scaling_factor)
+        key = ("rope_angles", self.base, self.rotary_dim, self.scaling_factor,
+               tuple(sorted(self.long_waves.items())) if self.long_waves else None)
         table = batch.shared.get(key)
         if table is None:
             table = batch.shared[key] = kernels.rope_angles(batch.positions, self.inv_freq, batch.num_tokens)
