@@ -23,7 +23,7 @@
 //                   weights are the eight consecutive positions 8g .. 8g + 7 and its V^T operand one 16-byte read.
 // The softmax is online over steps of 32 positions that start at multiples of 32, so a token's
 // arithmetic depends on its position and the cache only.
-#include "common.h"
+#include "attn_extras.h"
 #include "pipeline.h"
 
 #ifndef HDP
@@ -158,7 +158,8 @@ __device__ __forceinline__ void load_step(int kb, int begin, int end, const Cach
 // unrolling): a wave has few steps and memory is the bound.
 template <bool REGS, bool EXT = true>
 __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo, int col_pos, int begin, int end,
-                                             const CacheView& cv, float scale, float softcap, f32x4 (&o)[DT], float& m, float& l) {
+                                             const CacheView& cv, float scale, float softcap, f32x4 (&o)[DT], float& m, float& l,
+                                             int keep_first = 0, const float* rel_row = nullptr, int rel_far = 0) {
   const int lane = threadIdx.x & 63, lg = lane >> 4;
   const int first = begin & ~31;
   if (first >= end) return;
@@ -185,8 +186,9 @@ __device__ __forceinline__ void attend_range(const bf16x8 (&qf)[KS], int col_lo,
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int p = kb + lg * 8 + sub * 4 + j;
-        const bool visible = p >= col_lo && p <= col_pos && p >= begin && p < end;
-        const float x = visible ? (EXT ? capped(s[sub][j] * scale, softcap) : s[sub][j] * scale) : -INFINITY;
+        const bool visible = (p >= col_lo || (EXT && p < keep_first)) && p <= col_pos && p >= begin && p < end;
+        float x = visible ? (EXT ? capped(s[sub][j] * scale, softcap) : s[sub][j] * scale) : -INFINITY;
+        if (EXT && rel_row) x += rel_row[min(max(col_pos - p, 0), rel_far)];   // a masked score stays -inf
         sv[sub * 4 + j] = x;
         tile_max = fmaxf(tile_max, x);
       }
@@ -237,6 +239,21 @@ __device__ __forceinline__ void load_q(const __bf16* qrow, int hd, bf16x8 (&qf)[
 // the banks only in part (such reads measured at 0.7 of the LDS rate). This kernel takes every head width
 // and page size; widths of 64, 128 and 256 that fill their padded width, with pages that divide 64, take
 // attn_prefill_direct_kernel below, which swizzles instead of padding.
+constexpr int PT_KV_TILE = 64;
+// The order in which a workgroup of a prompt kernel walks tiles of 64 positions: tile i of the walk starts at
+// 64 i below `kept` tiles, and at first + 64 (i - kept) from there on, where `first` is the tile of the first position
+// that the workgroup's first column sees through its window and `kept` tiles (none without kept first positions, and
+// none that the window's tiles hold anyway) cover the first positions that stay visible.
+struct TileWalk {
+  int first, kept;
+  __device__ __forceinline__ TileWalk(int window_begin, int keep_first) {
+    first = window_begin & ~(PT_KV_TILE - 1);
+    kept = min((keep_first + PT_KV_TILE - 1) / PT_KV_TILE, first / PT_KV_TILE);
+  }
+  __device__ __forceinline__ int at(int i) const { return i < kept ? i * PT_KV_TILE : first + (i - kept) * PT_KV_TILE; }
+  __device__ __forceinline__ int count(int end) const { return kept + (end - first + PT_KV_TILE - 1) / PT_KV_TILE; }
+};
+
 constexpr int PT_WAVES = 8;
 constexpr int PT_THREADS = PT_WAVES * 64;
 constexpr int PT_TOKENS = PT_WAVES * 16;   // tokens of a tile
@@ -252,7 +269,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, float softcap, int cus) {
+    float scale, int window, float softcap, int cus, AttnExtras ex) {
   extern __shared__ __attribute__((aligned(16))) __bf16 lds[];
   __bf16* sK = lds;                     // [PT_KV][PT_KROW]
   __bf16* sV = lds + PT_KV * PT_KROW;   // [HDP][PT_VROW]
@@ -275,7 +292,10 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // the workgroup's range of positions
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = first_pos + tile_off;
-  const int begin = first_visible(tile_first_pos, window);
+  // the tiles of 64 positions that the workgroup walks: those from the first position that its first column's window
+  // holds on, and before them the tiles of the first positions that stay visible whatever the window has passed
+  const TileWalk walk(first_visible(tile_first_pos, window), ex.keep_first);
+  const int begin = ex.keep_first > 0 ? 0 : first_visible(tile_first_pos, window);
   const int end = tile_first_pos + tile_cols;  // one past the last column's position
 
   // this wave's columns
@@ -398,6 +418,8 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   // first tiles.
   const float c2 = scale * 1.44269504088896341f;
   const float cap_raw = softcap > 0.f ? softcap / scale : 0.f, cap_inv = softcap > 0.f ? scale / softcap : 0.f;
+  const float* rel_row = ex.rel ? ex.rel + (size_t)h * (ex.rel_far + 1) : nullptr;
+  const float inv_scale = 1.f / scale;
   auto tile_body = [&](bool masked, int p0) {
     // ---- scores of four 16-position tiles
     f32x4 s[4];
@@ -417,6 +439,13 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[sub][j] = cap_raw * tanhf(s[sub][j] * cap_inv);
     }
+    if (rel_row) {   // the bias by distance, in units of the raw score
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          s[sub][j] = __builtin_fmaf(rel_row[min(max(col_pos - (p0 + sub * 16 + lg * 4 + j), 0), ex.rel_far)], inv_scale, s[sub][j]);
+    }
     // ---- mask, running max, weights
     if (masked) {
 #pragma unroll
@@ -424,7 +453,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int p = p0 + sub * 16 + lg * 4 + j;
-          if (!(p >= col_lo && p <= col_pos)) s[sub][j] = -INFINITY;
+          if (!((p >= col_lo || p < ex.keep_first) && p <= col_pos)) s[sub][j] = -INFINITY;
         }
     }
     float tile_max = -INFINITY;
@@ -469,19 +498,20 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
     }
   };
 
-  const int first_tile = begin & ~(PT_KV - 1);
-  lookup(first_tile);
-  fetch(first_tile);
-  lookup(first_tile + PT_KV);
+  const int all_tiles = walk.count(end);
+  lookup(walk.at(0));
+  fetch(walk.at(0));
+  lookup(walk.at(1));
   stash();
   __syncthreads();
-  for (int p0 = first_tile; p0 < end; p0 += PT_KV) {
-    const bool more = p0 + PT_KV < end;
+  for (int i = 0; i < all_tiles; ++i) {
+    const int p0 = walk.at(i);
+    const bool more = i + 1 < all_tiles;
     if (more) {
-      fetch(p0 + PT_KV);        // with the page ids looked up one tile ago
-      lookup(p0 + 2 * PT_KV);
+      fetch(walk.at(i + 1));        // with the page ids looked up one tile ago
+      lookup(walk.at(i + 2));
     }
-    if (p0 < wave_end && p0 + PT_KV > wave_begin)   // some of this tile is visible to this wave
+    if (p0 < wave_end && (p0 + PT_KV > wave_begin || p0 < ex.keep_first))   // some of this tile is visible to this wave
       tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0);
     __syncthreads();  // everyone is done with this tile
     if (more) {
@@ -491,6 +521,7 @@ __global__ __launch_bounds__(PT_THREADS) void attn_prefill_kernel(
   }
   l = sum_of_column(l);
   if (!col_ok) return;
+  if (ex.sink) l += __builtin_amdgcn_exp2f(__builtin_fmaf(ex.sink[h], 1.44269504088896341f, -m * c2));   // m is a raw score
   const float inv = 1.f / l;
   __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
 #pragma unroll
@@ -556,7 +587,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     const __bf16* __restrict__ v_cache, __bf16* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, float scale,
-    int window, float softcap, int cus, float* __restrict__ partial, int chunk_tiles, int max_chunks) {
+    int window, float softcap, int cus, float* __restrict__ partial, int chunk_tiles, int max_chunks, AttnExtras ex) {
   static_assert(!(SPLIT && CHUNKED), "a chunk is taken by a workgroup of eight waves");
   typedef __attribute__((address_space(3))) void* lds_ptr;
   typedef __attribute__((address_space(1))) const void* global_ptr;
@@ -598,10 +629,10 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = first_pos + tile_off;
-  const int begin = first_visible(tile_first_pos, window);
+  const TileWalk walk(first_visible(tile_first_pos, window), ex.keep_first);   // as in attn_prefill_kernel
+  const int begin = ex.keep_first > 0 ? 0 : first_visible(tile_first_pos, window);
   const int end = tile_first_pos + tile_cols;
-  const int first_tile = begin & ~(PT_KV - 1);
-  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
+  const int all_tiles = walk.count(end);
   const int chunks = CHUNKED ? (all_tiles + chunk_tiles - 1) / chunk_tiles : 1;
   if (CHUNKED && chunk >= chunks) return;   // the whole workgroup, before any barrier
 
@@ -683,6 +714,8 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 
   const float c2 = scale * 1.44269504088896341f;
   const float cap_raw = softcap > 0.f ? softcap / scale : 0.f, cap_inv = softcap > 0.f ? scale / softcap : 0.f;
+  const float* rel_row = ex.rel ? ex.rel + (size_t)h * (ex.rel_far + 1) : nullptr;
+  const float inv_scale = 1.f / scale;
   auto tile_body = [&](bool masked, int p0, const unsigned char* base) {
     // ---- scores: tile sub = 2 st + t holds positions p0 + 32 st + 8 g + 4 t + j in register j of lane group g
     f32x4 s[4];
@@ -702,13 +735,21 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
 #pragma unroll
         for (int j = 0; j < 4; ++j) s[sub][j] = cap_raw * tanhf(s[sub][j] * cap_inv);
     }
+    if (rel_row) {   // the bias by distance, in units of the raw score
+#pragma unroll
+      for (int sub = 0; sub < 4; ++sub)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          s[sub][j] = __builtin_fmaf(rel_row[min(max(col_pos - (p0 + (sub >> 1) * 32 + lg * 8 + (sub & 1) * 4 + j), 0), ex.rel_far)],
+                                     inv_scale, s[sub][j]);
+    }
     if (masked) {
 #pragma unroll
       for (int sub = 0; sub < 4; ++sub)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int p = p0 + (sub >> 1) * 32 + lg * 8 + (sub & 1) * 4 + j;
-          if (!(p >= col_lo && p <= col_pos)) s[sub][j] = -INFINITY;
+          if (!((p >= col_lo || p < ex.keep_first) && p <= col_pos)) s[sub][j] = -INFINITY;
         }
     }
     float tile_max = -INFINITY;
@@ -758,20 +799,20 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
   // same number of barriers)
   const int steps = CHUNKED ? min(chunk_tiles, all_tiles - chunk * chunk_tiles) : SPLIT ? (all_tiles + 1) / 2 : all_tiles;
   const int my_tiles = half ? all_tiles - steps : steps;
-  const int my_first = first_tile + (CHUNKED ? chunk * chunk_tiles * PT_KV : half ? steps * PT_KV : 0);
-  lookup(my_first);
+  const int my_first = CHUNKED ? chunk * chunk_tiles : half ? steps : 0;   // in tiles of the walk
+  lookup(walk.at(my_first));
   if (my_tiles > 0) issue(0);
-  lookup(my_first + PT_KV);
+  lookup(walk.at(my_first + 1));
   wait_own_loads();
   __syncthreads();
   int stage = 0;
   for (int i = 0; i < steps; ++i) {
-    const int p0 = my_first + i * PT_KV;
+    const int p0 = walk.at(my_first + i);
     if (i + 1 < my_tiles) {
       issue(stage ^ 1);            // nobody reads that stage any more: the barrier that ended the last tile
-      lookup(p0 + 2 * PT_KV);
+      lookup(walk.at(my_first + i + 2));
     }
-    if (i < my_tiles && p0 < wave_end && p0 + PT_KV > wave_begin)
+    if (i < my_tiles && p0 < wave_end && (p0 + PT_KV > wave_begin || p0 < ex.keep_first))
       tile_body(!(p0 + PT_KV - 1 <= wave_first && p0 >= wave_lo_max), p0, lds_half + stage * PD_STAGE);
     wait_own_loads();   // a barrier alone does not wait for loads that write LDS
     __syncthreads();
@@ -796,6 +837,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     l = l * a0 + l1 * a1;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[dt] = o[dt] * a0 + hand_o[(wave * DT + dt) * 64 + lane] * a1;
+    m = m_both;   // what the sums are now relative to (a sink is weighed against it below)
   }
   l = sum_of_column(l);
   if (!col_ok) return;
@@ -809,6 +851,7 @@ __global__ __launch_bounds__(SPLIT ? 2 * PT_THREADS : PT_THREADS) void attn_pref
     }
     return;
   }
+  if (ex.sink) l += __builtin_amdgcn_exp2f(__builtin_fmaf(ex.sink[h], 1.44269504088896341f, -m * c2));   // m is a raw score
   const float inv = 1.f / l;
   __bf16* dst = out + (size_t)(tok0 + c) * heads * hd + (size_t)h * hd;
 #pragma unroll
@@ -829,17 +872,17 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
                                                                  const int* __restrict__ tiles,
                                                                  const int* __restrict__ entry_start,
                                                                  const int* __restrict__ entry_first_pos, int heads,
-                                                                 float scale, int window, float softcap, int chunk_tiles, int max_chunks) {
+                                                                 float scale, int window, float softcap, int chunk_tiles, int max_chunks,
+                                                                 AttnExtras ex) {
   constexpr int hd = HDP, QUADS = HDP / 4, AHEAD = 4;
   const int tile = blockIdx.x, h = blockIdx.y;
   const int entry = tiles[2 * tile], tile_off = tiles[2 * tile + 1];
   const int tok0 = entry_start[entry], count = entry_start[entry + 1] - tok0;
   const int tile_cols = min(PT_TOKENS, count - tile_off);
   const int tile_first_pos = entry_first_pos[entry] + tile_off;
-  const int begin = first_visible(tile_first_pos, window);
+  const TileWalk walk(first_visible(tile_first_pos, window), ex.keep_first);
   const int end = tile_first_pos + tile_cols;
-  const int first_tile = begin & ~(PT_KV - 1);
-  const int all_tiles = (end - first_tile + PT_KV - 1) / PT_KV;
+  const int all_tiles = walk.count(end);
   const int chunks = (all_tiles + chunk_tiles - 1) / chunk_tiles;
   if (chunks <= 1) return;
   const int at = blockIdx.z * 256 + threadIdx.x;
@@ -871,6 +914,7 @@ __global__ __launch_bounds__(256) void attn_prefill_merge_kernel(const float* __
         best = both;
       }
   }
+  if (ex.sink) total += __builtin_amdgcn_exp2f(__builtin_fmaf(ex.sink[h], 1.44269504088896341f, -best * c2));
   const float inv = 1.f / total;
   bf16x4 r;
 #pragma unroll
@@ -904,7 +948,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
     const __bf16* __restrict__ v_cache, float* __restrict__ partial, __bf16* __restrict__ out,
     const int* __restrict__ entries, const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, float softcap, int chunk, int head_blocks, int dense) {
+    float scale, int window, float softcap, int chunk, int head_blocks, int dense, AttnExtras ex) {
   const int lane = threadIdx.x & 63, lr = lane & 15, lg = lane >> 4;
   const int wave = JOINED ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : 0;
   const int chunk_index = JOINED ? wave : blockIdx.z, chunks = JOINED ? (int)(blockDim.x >> 6) : (int)gridDim.z;
@@ -921,7 +965,9 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
     early_pages = block_table[(size_t)entry * table_width + min(ps.page(chunk_index * chunk) + lane, table_width - 1)];
   const int pos = entry_first_pos[entry];
   const int lo = EXT ? first_visible(pos, window) : ((window > 0 && pos + 1 > window) ? pos + 1 - window : 0);
-  const int begin = max(lo, chunk_index * chunk), end = min(pos + 1, (chunk_index + 1) * chunk);
+  // a chunk that holds kept first positions starts with them; what lies between them and the window is masked
+  const int begin = (EXT && chunk_index * chunk < ex.keep_first) ? chunk_index * chunk : max(lo, chunk_index * chunk);
+  const int end = min(pos + 1, (chunk_index + 1) * chunk);
   const int head_in_group = hb * 16 + lr;
   const bool col_ok = head_in_group < group;
   const int h = kvh * group + head_in_group;
@@ -947,7 +993,8 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
       const int index = cv.page0 + lane;
       if (index <= ps.page(end - 1) && index < table_width) cv.pages = cv.table[index];
     }
-    attend_range<REGS, EXT>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, softcap, o, m, l);
+    attend_range<REGS, EXT>(qf, lo, col_ok ? pos : -1, begin, end, cv, scale, softcap, o, m, l, ex.keep_first,
+                            (EXT && ex.rel && col_ok) ? ex.rel + (size_t)h * (ex.rel_far + 1) : nullptr, ex.rel_far);
     l = sum_of_column(l);
   }
   if constexpr (JOINED) {
@@ -969,6 +1016,7 @@ __global__ __launch_bounds__(JOINED ? JOINED_WAVES * 64 : 64) __attribute__((amd
       const float mc = max_sum[(c * 16 + lr) * 2];
       total += (mc > -INFINITY ? __expf(mc - best) : 0.f) * max_sum[(c * 16 + lr) * 2 + 1];
     }
+    if (EXT && ex.sink && col_ok) total += __expf(ex.sink[h] - best);
     const float inv = 1.f / total;
     for (int dt = wave; dt < DT; dt += chunks) {
       f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -1011,7 +1059,7 @@ __global__ __launch_bounds__(CB_THREADS) void attn_combine_kernel(const float* _
                                                                   __bf16* __restrict__ out,
                                                                   const int* __restrict__ entries,
                                                                   const int* __restrict__ entry_start, int heads, int hd,
-                                                                  int chunks) {
+                                                                  int chunks, const float* __restrict__ sink) {
   __shared__ float weight[MAX_CHUNKS];
   __shared__ float wave_best[4], wave_total[4];
   __shared__ f32x4 part_sum[CB_THREADS];
@@ -1042,7 +1090,8 @@ __global__ __launch_bounds__(CB_THREADS) void attn_combine_kernel(const float* _
   const float mine = wave_sum(w * lc);
   if (lane == 0) wave_total[wave] = mine;
   __syncthreads();
-  const float inv = 1.f / (((wave_total[0] + wave_total[1]) + wave_total[2]) + wave_total[3]);
+  const float inv = 1.f / ((((wave_total[0] + wave_total[1]) + wave_total[2]) + wave_total[3])
+                           + (sink ? __expf(sink[h] - best) : 0.f));
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   if (active) {
     int c = part;
@@ -1082,12 +1131,16 @@ extern "C" int vk_attn_bf16_hdp() { return HDP; }
 // chunk_tiles > 0 (with the kernel that loads straight into LDS; ignored otherwise): a tile's steps of 64 positions
 // are cut into chunks of that many, a workgroup each, of which no tile has more than `max_chunks`; `partial` holds
 // num_tiles * heads * max_chunks * 128 * (padded head width + 4) floats.
-extern "C" int vk_attn_bf16_prefill_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+// sink, rel, rel_far, keep_first: see attn_extras.h (null, null, 0, 0: none of them).
+extern "C" int vk_attn_bf16_prefill_ext(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                     void* out, const int* tiles, int num_tiles, const int* entry_start,
                                     const int* entry_first_pos, const int* block_table, int table_width,
                                     int block_size, int heads, int kv_heads, int hd, float scale, int window, float softcap,
                                     int split, float* partial, long long partial_floats, int chunk_tiles,
-                                    int max_chunks, void* stream) {
+                                    int max_chunks, const float* sink, const float* rel, int rel_far, int keep_first,
+                                    void* stream) {
+  const AttnExtras ex{sink, rel, rel_far, keep_first};
+  if (rel_far < 0 || keep_first < 0 || (keep_first > 0 && window <= 0)) return VK_BAD_ARGUMENT;
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7))
@@ -1128,10 +1181,10 @@ extern "C" int vk_attn_bf16_prefill_capped(const void* q, long long q_stride, co
     chunked<<<num_tiles * heads * max_chunks, PT_THREADS, 2 * PD_STAGE, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
         entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, cus, partial,
-        chunk_tiles, max_chunks);
+        chunk_tiles, max_chunks, ex);
     VK_LAUNCH_CHECK();
     attn_prefill_merge_kernel<<<dim3(num_tiles, heads, PT_TOKENS * (HDP / 4) / 256), 256, 0, (hipStream_t)stream>>>(
-        partial, (__bf16*)out, tiles, entry_start, entry_first_pos, heads, scale, window, softcap, chunk_tiles, max_chunks);
+        partial, (__bf16*)out, tiles, entry_start, entry_first_pos, heads, scale, window, softcap, chunk_tiles, max_chunks, ex);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -1150,27 +1203,41 @@ extern "C" int vk_attn_bf16_prefill_capped(const void* q, long long q_stride, co
     }
     direct<<<num_tiles * heads, halves ? 2 * PT_THREADS : PT_THREADS, direct_lds, (hipStream_t)stream>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, cus, nullptr, 0, 1);
+        entry_first_pos, block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, cus, nullptr, 0, 1, ex);
     VK_LAUNCH_CHECK();
     return 0;
   }
 #endif
   kernel<<<num_tiles * heads, PT_THREADS, lds_bytes, (hipStream_t)stream>>>(
       (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, (__bf16*)out, tiles, entry_start,
-      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, cus);
+      entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, cus, ex);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_attn_bf16_prefill_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                    void* out, const int* tiles, int num_tiles, const int* entry_start,
+                                    const int* entry_first_pos, const int* block_table, int table_width,
+                                    int block_size, int heads, int kv_heads, int hd, float scale, int window, float softcap,
+                                    int split, float* partial, long long partial_floats, int chunk_tiles,
+                                    int max_chunks, void* stream) {
+  return vk_attn_bf16_prefill_ext(q, q_stride, k_cache, v_cache, out, tiles, num_tiles, entry_start, entry_first_pos,
+                                  block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, split,
+                                  partial, partial_floats, chunk_tiles, max_chunks, nullptr, nullptr, 0, 0, stream);
 }
 
 // entries: indices of the step's entries that hold exactly one token. partial: at least
 // num_entries * heads * chunks * (hd + 2) floats. `chunks` must cover the longest visible range:
 // chunks * chunk >= longest position + 1. `join` nonzero: one workgroup of `chunks` waves (at most 8) per entry and
 // key head merges its chunks itself and writes `out`; `partial` is not used and may be null.
-extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+extern "C" int vk_attn_bf16_decode_ext(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
                                    void* out, float* partial, const int* entries, int num_entries,
                                    const int* entry_start, const int* entry_first_pos, const int* block_table,
                                    int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                   int window, float softcap, int chunk, int chunks, int dense, int join, void* stream) {
+                                   int window, float softcap, int chunk, int chunks, int dense, int join,
+                                   const float* sink, const float* rel, int rel_far, int keep_first, void* stream) {
+  const AttnExtras ex{sink, rel, rel_far, keep_first};
+  if (rel_far < 0 || keep_first < 0 || (keep_first > 0 && window <= 0)) return VK_BAD_ARGUMENT;
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > HDP || (hd & 7) || block_size <= 0 || (block_size & 7) || heads <= 0 || kv_heads <= 0 ||
       heads % kv_heads || (q_stride & 7) || chunk < 32 || (chunk & 31) || chunks <= 0 ||
@@ -1181,7 +1248,7 @@ extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, con
   const int group = heads / kv_heads, head_blocks = (group + 15) / 16;
   if (kv_heads * head_blocks > 65535 || heads > 65535) return VK_UNSUPPORTED_SIZE;
   hipStream_t s = (hipStream_t)stream;
-  const bool ext = softcap > 0.f || window < 0;
+  const bool ext = softcap > 0.f || window < 0 || sink || rel || keep_first > 0;
   // pages a chunk can touch: chunks start at multiples of `chunk`, which need not be page edges
   const int chunk_pages = chunk % block_size == 0 ? chunk / block_size : chunk / block_size + 2;
   if (join) {
@@ -1199,7 +1266,7 @@ extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, con
     kernel<<<dim3(num_entries, kv_heads * head_blocks), chunks * 64, lds_bytes, s>>>(
         (const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, nullptr, (__bf16*)out, entries,
         entry_start, entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, chunk,
-        head_blocks, dense);
+        head_blocks, dense, ex);
     VK_LAUNCH_CHECK();
     return 0;
   }
@@ -1208,12 +1275,22 @@ extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, con
                     : (chunk_pages <= 64 ? attn_decode_kernel<true, false, false> : attn_decode_kernel<false, false, false>);
   kernel<<<grid, 64, 0, s>>>((const __bf16*)q, q_stride, (const __bf16*)k_cache, (const __bf16*)v_cache, partial,
                              (__bf16*)out, entries, entry_start, entry_first_pos, block_table, table_width, block_size,
-                             heads, kv_heads, hd, scale, window, softcap, chunk, head_blocks, dense);
+                             heads, kv_heads, hd, scale, window, softcap, chunk, head_blocks, dense, ex);
   VK_LAUNCH_CHECK();
   dim3 cgrid(num_entries, heads);
-  attn_combine_kernel<<<cgrid, CB_THREADS, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks);
+  attn_combine_kernel<<<cgrid, CB_THREADS, 0, s>>>(partial, (__bf16*)out, entries, entry_start, heads, hd, chunks, sink);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_attn_bf16_decode_capped(const void* q, long long q_stride, const void* k_cache, const void* v_cache,
+                                   void* out, float* partial, const int* entries, int num_entries,
+                                   const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                   int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                   int window, float softcap, int chunk, int chunks, int dense, int join, void* stream) {
+  return vk_attn_bf16_decode_ext(q, q_stride, k_cache, v_cache, out, partial, entries, num_entries, entry_start,
+                                 entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window,
+                                 softcap, chunk, chunks, dense, join, nullptr, nullptr, 0, 0, stream);
 }
 
 // The same two without a cap on the scores.

@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
     const float* __restrict__ v_cache, float* __restrict__ partial, const int* __restrict__ entries,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos,
     const int* __restrict__ block_table, int table_width, int block_size, int heads, int kv_heads, int hd,
-    float scale, int window, float softcap, int head_blocks) {
+    float scale, int window, float softcap, int head_blocks, AttnExtras ex) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   __shared__ float sw[4][HB][DEC_WAVE];                 // a wave's scores, then its weights
   __shared__ float merge_o[4][HB][MAX_HD];              // the waves' weighted sums
@@ -140,7 +140,8 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
   const size_t stride = hd + 2;
   float* dst = partial + (((size_t)slot_index * heads + first_head) * gridDim.z + blockIdx.z) * stride;
   const size_t head_stride = (size_t)gridDim.z * stride;
-  if (chunk_begin > pos || chunk_begin + DEC_CHUNK <= lo) {           // nothing of this chunk is visible
+  const int keep = ex.keep_first;                                     // positions below it stay visible
+  if (chunk_begin > pos || (chunk_begin + DEC_CHUNK <= lo && chunk_begin >= keep)) {   // nothing of this chunk is visible
     if ((int)threadIdx.x < block_heads) {
       dst[threadIdx.x * head_stride + hd] = -INFINITY;
       dst[threadIdx.x * head_stride + hd + 1] = 0.f;
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
   }
   const int* table = block_table + (size_t)entry * table_width;
   const int wave_begin = chunk_begin + wave * DEC_WAVE;
-  const bool wave_sees = wave_begin <= pos && wave_begin + DEC_WAVE > lo;
+  const bool wave_sees = wave_begin <= pos && (wave_begin + DEC_WAVE > lo || wave_begin < keep);
 
   // ---- scores
   const int ps = lane >> 4, c = lane & 15;
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
 #pragma unroll
       for (int b = 0; b < AHEAD; ++b) {
         const int p = wave_begin + (it0 + b) * 4 + ps;
-        at[b] = min(max(p, lo), pos);   // a position outside the range reads one inside it; its score is masked
+        at[b] = p < keep ? min(p, pos) : min(max(p, lo), pos);   // a position outside the range reads one inside it; its score is masked
         page[b] = table[at[b] / block_size];
       }
       f32x4 k4[AHEAD][QC];
@@ -202,7 +203,11 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
         for (int h = 0; h < HB; ++h) {
 #pragma unroll
           for (int off = 1; off < 16; off <<= 1) dot[h] += __shfl_xor(dot[h], off, WAVE);
-          if (c == 0) sw[wave][h][(it0 + b) * 4 + ps] = (p >= lo && p <= pos) ? capped(dot[h] * scale, softcap) : -INFINITY;
+          if (c == 0) {
+            float sc = ((p >= lo || p < keep) && p <= pos) ? capped(dot[h] * scale, softcap) : -INFINITY;
+            if (ex.rel && h < block_heads) sc += distance_bias(ex, first_head + h, max(pos - p, 0));
+            sw[wave][h][(it0 + b) * 4 + ps] = sc;
+          }
         }
       }
     }
@@ -235,10 +240,10 @@ __global__ __launch_bounds__(256) void attn_decode_f32_kernel(
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int p0 = wave_begin + (qs + 4 * j) * 4;             // four positions of one page
-      const bool any = p0 <= pos && p0 + 3 >= lo;
+      const bool any = p0 <= pos && (p0 + 3 >= lo || p0 < keep);
       const int from = any ? p0 : (pos & ~3);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) sees[j][e] = any && p0 + e >= lo && p0 + e <= pos;
+      for (int e = 0; e < 4; ++e) sees[j][e] = any && (p0 + e >= lo || p0 + e < keep) && p0 + e <= pos;
       quad[j] = v_cache + ((size_t)table[from / block_size] * kv_heads + kvh) * hd * block_size + from % block_size;
     }
 #pragma unroll
@@ -307,7 +312,7 @@ template <typename T>
 __global__ __launch_bounds__(64) void attn_combine_f32_kernel(const float* __restrict__ partial, T* __restrict__ out,
                                                               const int* __restrict__ entries,
                                                               const int* __restrict__ entry_start, int heads, int hd,
-                                                              int chunks) {
+                                                              int chunks, AttnExtras ex) {
   const int slot_index = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const size_t stride = hd + 2;
   const float* src = partial + ((size_t)slot_index * heads + h) * chunks * stride;
@@ -325,7 +330,7 @@ __global__ __launch_bounds__(64) void attn_combine_f32_kernel(const float* __res
         sum = fmaf(src[(size_t)ch * stride + hd + 1], factor, sum);
       }
     }
-    out[(size_t)token * heads * hd + (size_t)h * hd + d] = from_float<T>(total / sum);
+    out[(size_t)token * heads * hd + (size_t)h * hd + d] = from_float<T>(total / (sum + sink_term(ex, h, best)));
   }
 }
 
@@ -353,7 +358,8 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     const float* __restrict__ q, long long q_stride, const float* __restrict__ k_cache,
     const float* __restrict__ v_cache, float* __restrict__ out, const int* __restrict__ tiles,
     const int* __restrict__ entry_start, const int* __restrict__ entry_first_pos, const int* __restrict__ block_table,
-    int table_width, int block_size, int heads, int kv_heads, float scale, int window, float softcap, int tile_tokens) {
+    int table_width, int block_size, int heads, int kv_heads, float scale, int window, float softcap, int tile_tokens,
+    AttnExtras ex) {
   typedef float f32x4 __attribute__((ext_vector_type(4)));
   constexpr int HD = 16 * DPT, QROW = HD + 4, VROW = PF_TILE + 4;
   extern __shared__ __attribute__((aligned(16))) float pf_lds[];
@@ -391,23 +397,29 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
     for (int j = 0; j < DPT; ++j) o[i][j] = 0.f;
   }
   const int lowest = first_visible(pos0, window);   // the first token's first position
-  for (int kv0 = lowest / PF_TILE * PF_TILE; kv0 <= last_pos; kv0 += PF_TILE) {
+  // the tiles of the first positions that stay visible whatever the window has passed come first (those that the
+  // window's own tiles do not hold anyway), then the tiles from the window's first position on
+  const int keep = ex.keep_first;
+  const int first_tile = lowest / PF_TILE, kept_tiles = min((keep + PF_TILE - 1) / PF_TILE, first_tile);
+  for (int it = 0;; ++it) {
+    const int kv0 = (it < kept_tiles ? it : first_tile + (it - kept_tiles)) * PF_TILE;
+    if (kv0 > last_pos) break;
     __syncthreads();   // the tile before has been read
     for (int i = tid; i < PF_TILE * (HD / 4); i += 256) {
       const int r = i / (HD / 4), c = (i % (HD / 4)) * 4, p = kv0 + r;
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if (p >= lowest && p <= last_pos)   // below `lowest` the window has passed: the page may have been given back
+      if ((p >= lowest || p < keep) && p <= last_pos)   // below `lowest` the window has passed: the page may have been given back
         v = *(const f32x4*)(k_cache + (((size_t)table[p / block_size] * kv_heads + kvh) * block_size + p % block_size) * HD + c);
       *(f32x4*)(k_s + r * QROW + c) = v;
     }
     for (int i = tid; i < HD * (PF_TILE / 4); i += 256) {
       const int d = i / (PF_TILE / 4), c = (i % (PF_TILE / 4)) * 4, p = kv0 + c;   // four positions of one page
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
-      if (p + 3 >= lowest && p <= last_pos) {   // the four share a page, which is held if any of them is visible
+      if ((p + 3 >= lowest || p < keep) && p <= last_pos) {   // the four share a page, which is held if any of them is visible
         v = *(const f32x4*)(v_cache + (((size_t)table[p / block_size] * kv_heads + kvh) * HD + d) * block_size + p % block_size);
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (p + e < lowest || p + e > last_pos) v[e] = 0.f;
+          if ((p + e < lowest && p + e >= keep) || p + e > last_pos) v[e] = 0.f;
       }
       *(f32x4*)(v_s + d * VROW + c) = v;
     }
@@ -451,8 +463,9 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const int p = kv0 + tx + 16 * j;
-        const bool sees = 4 * ty + i < rows && p <= qpos && p >= first;
+        const bool sees = 4 * ty + i < rows && p <= qpos && (p >= first || p < keep);
         s[i][j] = sees ? capped(s[i][j] * scale, softcap) : -INFINITY;
+        if (ex.rel && sees) s[i][j] += distance_bias(ex, h, qpos - p);
         best = fmaxf(best, s[i][j]);
       }
 #pragma unroll
@@ -501,8 +514,9 @@ __global__ __launch_bounds__(256) void attn_prefill_f32_kernel(
   for (int i = 0; i < 4; ++i) {
     if (4 * ty + i >= rows) continue;
     float* dst = out + (size_t)(tok0 + 4 * ty + i) * heads * HD + (size_t)h * HD;
+    const float whole = l[i] + sink_term(ex, h, m[i]);
 #pragma unroll
-    for (int j = 0; j < DPT; ++j) dst[tx + 16 * j] = o[i][j] / l[i];
+    for (int j = 0; j < DPT; ++j) dst[tx + 16 * j] = o[i][j] / whole;
   }
 }
 
@@ -510,7 +524,7 @@ template <int DPT>
 int launch_prefill_f32(dim3 grid, hipStream_t s, const float* q, long long q_stride, const float* k_cache,
                        const float* v_cache, float* out, const int* tiles, const int* entry_start,
                        const int* entry_first_pos, const int* block_table, int table_width, int block_size, int heads,
-                       int kv_heads, float scale, int window, float softcap, int tile_tokens) {
+                       int kv_heads, float scale, int window, float softcap, int tile_tokens, AttnExtras ex) {
   constexpr int HD = 16 * DPT;
   constexpr int lds_bytes = (2 * PF_TILE * (HD + 4) + HD * (PF_TILE + 4) + PF_TILE * (PF_TILE + 4)) * 4;
   static_assert(lds_bytes <= 160 * 1024, "a CU has 160 KB of LDS");
@@ -523,7 +537,7 @@ int launch_prefill_f32(dim3 grid, hipStream_t s, const float* q, long long q_str
   }
   attn_prefill_f32_kernel<DPT><<<grid, 256, lds_bytes, s>>>(q, q_stride, k_cache, v_cache, out, tiles, entry_start,
                                                             entry_first_pos, block_table, table_width, block_size,
-                                                            heads, kv_heads, scale, window, softcap, tile_tokens);
+                                                            heads, kv_heads, scale, window, softcap, tile_tokens, ex);
   return 0;
 }
 
@@ -531,10 +545,10 @@ template <int HB, int QC>
 void launch_decode_f32(dim3 grid, hipStream_t s, const float* q, long long q_stride, const float* k_cache,
                        const float* v_cache, float* partial, const int* entries, const int* entry_start,
                        const int* entry_first_pos, const int* block_table, int table_width, int block_size, int heads,
-                       int kv_heads, int hd, float scale, int window, float softcap, int head_blocks) {
+                       int kv_heads, int hd, float scale, int window, float softcap, int head_blocks, AttnExtras ex) {
   attn_decode_f32_kernel<HB, QC><<<grid, 256, 0, s>>>(q, q_stride, k_cache, v_cache, partial, entries, entry_start,
                                                       entry_first_pos, block_table, table_width, block_size, heads,
-                                                      kv_heads, hd, scale, window, softcap, head_blocks);
+                                                      kv_heads, hd, scale, window, softcap, head_blocks, ex);
 }
 }  // namespace
 
@@ -587,11 +601,14 @@ extern "C" int vk_attn_decode_f32_chunk() { return DEC_CHUNK; }
 
 // Attention of the single-token entries listed in `entries` in 32-bit: float q, cache and out. partial: at least
 // num_entries * heads * chunks * (hd + 2) floats; chunks * 256 >= longest position + 1.
-extern "C" int vk_attn_decode_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+extern "C" int vk_attn_decode_f32_ext(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
                                   float* out, float* partial, const int* entries, int num_entries,
                                   const int* entry_start, const int* entry_first_pos, const int* block_table,
                                   int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
-                                  int window, float softcap, int chunks, void* stream) {
+                                  int window, float softcap, int chunks, const float* sink, const float* rel, int rel_far,
+                                  int keep_first, void* stream) {
+  const AttnExtras ex{sink, rel, rel_far, keep_first};
+  if (!extras_ok(ex, window)) return VK_BAD_ARGUMENT;
   if (num_entries <= 0) return 0;
   if (hd <= 0 || hd > MAX_HD || (hd & 3) || block_size <= 0 || (block_size & 3) || (q_stride & 3)) return VK_UNSUPPORTED_SIZE;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || table_width <= 0 || chunks <= 0 ||
@@ -610,7 +627,7 @@ extern "C" int vk_attn_decode_f32_capped(const float* q, long long q_stride, con
   dim3 grid(num_entries, kv_heads * head_blocks, chunks);
 #define VK_DEC(HBV, QCV)                                                                                          \
   launch_decode_f32<HBV, QCV>(grid, s, q, q_stride, k_cache, v_cache, partial, entries, entry_start, entry_first_pos, \
-                              block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, head_blocks)
+                              block_table, table_width, block_size, heads, kv_heads, hd, scale, window, softcap, head_blocks, ex)
   if (qc == 1) {
     switch (hb) { case 1: VK_DEC(1, 1); break; case 2: VK_DEC(2, 1); break; case 4: VK_DEC(4, 1); break; default: VK_DEC(8, 1); }
   } else if (qc == 2) {
@@ -620,18 +637,31 @@ extern "C" int vk_attn_decode_f32_capped(const float* q, long long q_stride, con
   }
 #undef VK_DEC
   VK_LAUNCH_CHECK();
-  attn_combine_f32_kernel<float><<<dim3(num_entries, heads), 64, 0, s>>>(partial, out, entries, entry_start, heads, hd, chunks);
+  attn_combine_f32_kernel<float><<<dim3(num_entries, heads), 64, 0, s>>>(partial, out, entries, entry_start, heads, hd, chunks, ex);
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_attn_decode_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                  float* out, float* partial, const int* entries, int num_entries,
+                                  const int* entry_start, const int* entry_first_pos, const int* block_table,
+                                  int table_width, int block_size, int heads, int kv_heads, int hd, float scale,
+                                  int window, float softcap, int chunks, void* stream) {
+  return vk_attn_decode_f32_ext(q, q_stride, k_cache, v_cache, out, partial, entries, num_entries, entry_start,
+                                entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window,
+                                softcap, chunks, nullptr, nullptr, 0, 0, stream);
 }
 
 // Attention of the step's prompt portions in 32-bit: float q, cache and out. tiles: pairs (entry, first token of the
 // tile within the entry), `tile_tokens` tokens a tile (a multiple of 64), as vk_attn_bf16_prefill takes them. Head
 // widths that are multiples of 16 up to 128, pages of a multiple of 4 positions.
-extern "C" int vk_attn_prefill_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+extern "C" int vk_attn_prefill_f32_ext(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
                                    float* out, const int* tiles, int num_tiles, int tile_tokens, const int* entry_start,
                                    const int* entry_first_pos, const int* block_table, int table_width, int block_size,
-                                   int heads, int kv_heads, int hd, float scale, int window, float softcap, void* stream) {
+                                   int heads, int kv_heads, int hd, float scale, int window, float softcap,
+                                   const float* sink, const float* rel, int rel_far, int keep_first, void* stream) {
+  const AttnExtras ex{sink, rel, rel_far, keep_first};
+  if (!extras_ok(ex, window)) return VK_BAD_ARGUMENT;
   if (num_tiles <= 0) return 0;
   if (hd <= 0 || hd > 128 || (hd & 15) || block_size <= 0 || (block_size & 3) || (q_stride & 3)) return VK_UNSUPPORTED_SIZE;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || heads > 65535 || table_width <= 0 ||
@@ -646,13 +676,22 @@ extern "C" int vk_attn_prefill_f32_capped(const float* q, long long q_stride, co
 #define VK_PF(DPTV)                                                                                                  \
   case DPTV:                                                                                                         \
     status = launch_prefill_f32<DPTV>(grid, s, q, q_stride, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, \
-                                      block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, tile_tokens); \
+                                      block_table, table_width, block_size, heads, kv_heads, scale, window, softcap, tile_tokens, ex); \
     break;
   switch (hd / 16) { VK_PF(1) VK_PF(2) VK_PF(3) VK_PF(4) VK_PF(5) VK_PF(6) VK_PF(7) VK_PF(8) }
 #undef VK_PF
   if (status != 0) return status;
   VK_LAUNCH_CHECK();
   return 0;
+}
+
+extern "C" int vk_attn_prefill_f32_capped(const float* q, long long q_stride, const float* k_cache, const float* v_cache,
+                                   float* out, const int* tiles, int num_tiles, int tile_tokens, const int* entry_start,
+                                   const int* entry_first_pos, const int* block_table, int table_width, int block_size,
+                                   int heads, int kv_heads, int hd, float scale, int window, float softcap, void* stream) {
+  return vk_attn_prefill_f32_ext(q, q_stride, k_cache, v_cache, out, tiles, num_tiles, tile_tokens, entry_start,
+                                 entry_first_pos, block_table, table_width, block_size, heads, kv_heads, hd, scale, window,
+                                 softcap, nullptr, nullptr, 0, 0, stream);
 }
 
 // The same three without a cap on the scores.

@@ -136,10 +136,6 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
     becomes ``softcap * tanh(score / softcap)`` before the softmax.  ``extras``: see :class:`AttentionExtras`."""
     if extras is not None and not extras.any():
         extras = None
-    if extras is not None:
-        kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
-                             head_dim, scale, window, softcap=softcap, extras=extras)
-        return
     if kernels.attn_bf16_supported(qkv, k_cache, head_dim):
         if batch.num_prefill_tiles:
             cus = kernels.compute_units(qkv.device)
@@ -150,7 +146,7 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
                                                             batch.sum_tile_reach, cus)
             kernels.attn_bf16_prefill(qkv, k_cache, v_cache, out, batch.prefill_tiles, batch.entry_start,
                                       batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, split,
-                                      *(chunked or (0, 0)), softcap=softcap)
+                                      *(chunked or (0, 0)), softcap=softcap, extras=extras)
         if batch.num_decode_entries:
             group = heads // kv_heads
             visible = batch.max_decode_kv_len
@@ -164,7 +160,7 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
                                                     dtype=torch.float32, device=qkv.device)
             kernels.attn_bf16_decode(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
                                      batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunk,
-                                     chunks, dense=batch.all_single, join=join, softcap=softcap)
+                                     chunks, dense=batch.all_single, join=join, softcap=softcap, extras=extras)
         return
     # the 32-bit run: single tokens on the kernel that splits their positions into chunks and shares the reads among
     # the query heads of a key head, prompt portions on the kernel that walks the positions in LDS tiles; what
@@ -176,13 +172,14 @@ def paged_attention(qkv, k_cache, v_cache, out, batch, table, heads, kv_heads, h
         partial = torch.empty(batch.num_decode_entries * heads * chunks * (head_dim + 2), dtype=torch.float32,
                               device=qkv.device)
         kernels.attn_decode_f32(qkv, k_cache, v_cache, out, partial, batch.decode_entries, batch.entry_start,
-                                batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunks, softcap=softcap)
+                                batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window, chunks, softcap=softcap,
+                                extras=extras)
     if portions:
         kernels.attn_prefill_f32(qkv, k_cache, v_cache, out, batch.prefill_tiles, batch.prefill_tile_tokens,
                                  batch.entry_start, batch.entry_first_pos, table, heads, kv_heads, head_dim, scale, window,
-                                 softcap=softcap)
+                                 softcap=softcap, extras=extras)
     if (batch.num_decode_entries and not singles) or (batch.num_prefill_tiles and not portions):
         # the general kernel can leave out the single tokens, not the portions: those it then computes again
         kernels.attn_generic(qkv, k_cache, v_cache, out, batch.positions, batch.entry_of_token, table, heads, kv_heads,
                              head_dim, scale, window, skip_single_of=batch.entry_start if singles else None,
-                             softcap=softcap)
+                             softcap=softcap, extras=extras)

@@ -46,7 +46,7 @@ MODULES: Dict[str, tuple] = {
 
 # matrix-core attention: one module per padded head width, compiled when a model of that width runs
 for _width in range(32, 257, 32):
-    MODULES[f"attn_bf16_hd{_width}"] = ("hip", ["kernels/attn_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h"],
+    MODULES[f"attn_bf16_hd{_width}"] = ("hip", ["kernels/attn_bf16.hip"], ["kernels/common.h", "kernels/pipeline.h", "kernels/attn_extras.h"],
                                          [f"-DHDP={_width}"])
 
 _loaded: Dict[str, ctypes.CDLL] = {}

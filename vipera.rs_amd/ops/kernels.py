@@ -320,7 +320,7 @@ def attn_decode_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim: 
 def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                     partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                     entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
-                    head_dim: int, scale: float, window: int, chunks: int, softcap: float = 0.0) -> None:
+                    head_dim: int, scale: float, window: int, chunks: int, softcap: float = 0.0, extras=None) -> None:
     """32-bit attention of the single-token entries listed in ``entries``; their positions are split into
     ``chunks`` of :data:`ATTN_DECODE_F32_CHUNK`, which must cover the longest visible range."""
     _dev(q, k_cache, v_cache, out, partial, entries, entry_start, entry_first_pos, block_table)
@@ -338,11 +338,12 @@ def attn_decode_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
     _need(heads % kv_heads == 0 and chunks >= 1, "attention: heads must be a multiple of kv_heads")
-    fn = _fn("attn_generic", "vk_attn_decode_f32_capped",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p])
+    fn = _fn("attn_generic", "vk_attn_decode_f32_ext",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p, _p, _i, _i, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
-               heads, kv_heads, head_dim, float(scale), int(window), float(softcap), int(chunks), _stream()), "attn_decode_f32")
+               heads, kv_heads, head_dim, float(scale), int(window), float(softcap), int(chunks),
+               *attn_extras_args(extras, heads, window), _stream()), "attn_decode_f32")
 
 
 ATTN_PREFILL_F32_MAX_HEAD_DIM = 128   # the K, V and weight tiles of a wider head do not fit a CU's LDS
@@ -359,7 +360,7 @@ def attn_prefill_f32_supported(q: torch.Tensor, k_cache: torch.Tensor, head_dim:
 def attn_prefill_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, out: torch.Tensor,
                      tiles: torch.Tensor, tile_tokens: int, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                      block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
-                     window: int, softcap: float = 0.0) -> None:
+                     window: int, softcap: float = 0.0, extras=None) -> None:
     """32-bit attention of the entries' tiles listed in ``tiles`` (pairs: entry, first token within it; ``tile_tokens``
     tokens a tile, a multiple of 64): 64 tokens of one head a workgroup, the positions in LDS tiles of 64."""
     _dev(q, k_cache, v_cache, out, tiles, entry_start, entry_first_pos, block_table)
@@ -375,11 +376,12 @@ def attn_prefill_f32(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
           and entry_start.numel() == block_table.shape[0] + 1 and entry_first_pos.numel() == block_table.shape[0],
           "attention: entry arrays")
     _need(heads % kv_heads == 0, "attention: heads must be a multiple of kv_heads")
-    fn = _fn("attn_generic", "vk_attn_prefill_f32_capped",
-             [_p, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _p])
+    fn = _fn("attn_generic", "vk_attn_prefill_f32_ext",
+             [_p, _ll, _p, _p, _p, _p, _i, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _p, _p, _i, _i, _p])
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), tiles.numel() // 2,
                int(tile_tokens), _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1],
-               k_cache.shape[2], heads, kv_heads, head_dim, float(scale), int(window), float(softcap), _stream()), "attn_prefill_f32")
+               k_cache.shape[2], heads, kv_heads, head_dim, float(scale), int(window), float(softcap),
+               *attn_extras_args(extras, heads, window), _stream()), "attn_prefill_f32")
 
 
 # ----------------------------------------------------------------------------------------------
@@ -752,7 +754,7 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       tiles: torch.Tensor, entry_start: torch.Tensor, entry_first_pos: torch.Tensor,
                       block_table: torch.Tensor, heads: int, kv_heads: int, head_dim: int, scale: float,
                       window: int, split: bool = False, chunk_tiles: int = 0, max_chunks: int = 0,
-                      softcap: float = 0.0) -> None:
+                      softcap: float = 0.0, extras=None) -> None:
     """Attention of the entries' 128-token tiles listed in ``tiles`` (pairs: entry, first token within it).
     ``split``: workgroups of sixteen waves that halve a tile's positions between them and merge at the end, where
     the kernel in use has that form (for few tiles of very different lengths); the same result up to rounding.
@@ -777,13 +779,14 @@ def attn_bf16_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     else:
         chunk_tiles = max_chunks = 0
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_prefill_capped",
-             [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p, _ll, _i, _i, _p],
+    fn = _fn(module, "vk_attn_bf16_prefill_ext",
+             [_p, _ll, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _p, _ll, _i, _i, _p, _p, _i, _i, _p],
              key=module + ".prefill")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(tiles), num_tiles,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
                heads, kv_heads, head_dim, float(scale), int(window), float(softcap), 1 if split else 0, _ptr(partial),
-               partial.numel() if partial is not None else 0, int(chunk_tiles), int(max_chunks), _stream()),
+               partial.numel() if partial is not None else 0, int(chunk_tiles), int(max_chunks),
+               *attn_extras_args(extras, heads, window), _stream()),
             "attn_bf16_prefill")
 
 
@@ -794,7 +797,7 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      partial: torch.Tensor, entries: torch.Tensor, entry_start: torch.Tensor,
                      entry_first_pos: torch.Tensor, block_table: torch.Tensor, heads: int, kv_heads: int,
                      head_dim: int, scale: float, window: int, chunk: int, chunks: int, dense: bool = False,
-                     join: bool = False, softcap: float = 0.0) -> None:
+                     join: bool = False, softcap: float = 0.0, extras=None) -> None:
     """Attention of the single-token entries listed in ``entries``, positions split into ``chunks`` of ``chunk``.
     ``dense``: the step holds single-token entries only, so entry i is the i-th of them and holds token i; the
     kernel then need not look either up.  ``join``: one workgroup per entry and key head takes all chunks (at most
@@ -815,12 +818,13 @@ def attn_bf16_decode(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _need(chunk >= 32 and chunk % 32 == 0 and chunks >= 1, "attention: chunk must be a multiple of 32")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(), "attention: table")
     module = f"attn_bf16_hd{attn_bf16_padded_width(head_dim)}"
-    fn = _fn(module, "vk_attn_bf16_decode_capped",
-             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _i, _i, _i, _p], key=module + ".decode")
+    fn = _fn(module, "vk_attn_bf16_decode_ext",
+             [_p, _ll, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _f, _i, _i, _i, _i, _p, _p, _i, _i, _p],
+             key=module + ".decode")
     _status(fn(_ptr(q), q.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(partial), _ptr(entries), count,
                _ptr(entry_start), _ptr(entry_first_pos), _ptr(block_table), block_table.shape[1], k_cache.shape[2],
                heads, kv_heads, head_dim, float(scale), int(window), float(softcap), int(chunk), int(chunks), 1 if dense else 0,
-               1 if join else 0, _stream()),
+               1 if join else 0, *attn_extras_args(extras, heads, window), _stream()),
             "attn_bf16_decode")
 
 
