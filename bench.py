@@ -106,7 +106,7 @@ def main() -> int:
                         help="also run one decode step (of --batch requests at --ctx) and one prefill eagerly with a "
                              "pair of GPU events around every kernel launch, and add the microseconds of each class of "
                              "kernel to the line (split_decode_us, split_prefill_us)")
-    parser.add_argument("--design", default="", choices=["", "gilidra", "zulesun", "muzasun"],
+    parser.add_argument("--design", default="", choices=["", "gilidra", "zulesun", "muzasun", "lurirax"],
                         help="instead of the headline measurement: prefill and decode of this design at layer sizes that "
                              "resemble a real model's (--size), beside the dense Qwen2 decoder of the same width, depth and "
                              "active feed-forward width, each with the time of every class of kernel")
@@ -443,6 +443,38 @@ def muzasun_shape(z):
             "residual_mult": 0.5, "logit_scale": 0.5, "layers": layers}
 
 
+def lurirax_shape(z):
+    """A Lurirax configuration of sizes ``z``: differential attention with kept first positions, twice attention in a
+    sliding window with a sink, attention within chunks with a bias by distance beside retention, a window again, and so
+    on; a dense feed-forward behind the differential layers and a mixture of experts with a gated shared expert behind
+    the others."""
+    heads, kv = z["heads"], max(1, z["heads"] // 4)
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"], "top": z["top"], "scale": 2.5},
+           "shared": {"ff": z["ff"]}}
+    dense = {"kind": "dense", "ff": z["top"] * z["ff"]}
+    window = {"heads": heads, "kv_heads": kv, "dim": z["dim"], "vdim": z["dim"], "mask": {"size": z["window"]},
+              "rot": {"base": 1e6, "dims": z["dim"] // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
+              "scale": z["dim"] ** -0.5}
+    two = {"heads": heads, "kv_heads": kv, "dim": z["dim"] // 2, "vdim": z["dim"], "diff": 0.5,
+           "mask": {"size": z["window"], "keep_first": 64}, "scale": (z["dim"] // 2) ** -0.5}
+    pair = {"left": {"heads": heads, "kv_heads": kv, "dim": z["dim"], "vdim": z["dim"], "mask": {"size": z["window"]},
+                     "bias_max": z["window"], "bias_rows": 32, "scale": z["dim"] ** -0.5},
+            "left_scale": 0.6, "right_scale": 0.5,
+            "right": {"heads": heads, "dim": z["dim"], "vdim": z["dim"], "rot": {"base": 1e6, "dims": z["dim"]},
+                      "decay": [1.0 - 2.0 ** (-1.0 - 7.0 * h / max(1, heads - 1)) for h in range(heads)]}}
+    layers = []
+    for index in range(z["layers"]):
+        kind = index % 5
+        if kind == 0:
+            layers.append({"type": "attention_2", "mixer": two, "mlp": dense})
+        elif kind == 3:
+            layers.append({"type": "parallel", "mixer": pair, "mlp": moe})
+        else:
+            layers.append({"type": "attention", "mixer": window, "mlp": moe})
+    return {"architecture": "Lurirax", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
+            "embedding": {"scale": 0.5}, "layers": layers}
+
+
 def dense_shape(z):
     """The dense Qwen2 decoder of the same width, depth, heads and active feed-forward width."""
     return dict(QWEN25_7B, num_hidden_layers=z["layers"], hidden_size=z["width"], num_attention_heads=z["heads"],
@@ -476,6 +508,8 @@ def design_comparison(args) -> int:
     runs = ((("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))) if args.design == "gilidra" else
             (("muzasun", muzasun_shape(z)), ("gilidra", gilidra_shape(z)), ("dense", dense_shape(z)))
             if args.design == "muzasun" else
+            (("lurirax", lurirax_shape(z)), ("zulesun", zulesun_shape(z)), ("dense", dense_shape(z)))
+            if args.design == "lurirax" else
             (("zulesun", zulesun_shape(z)), ("gilidra", gilidra_shape(z)), ("dense", dense_shape(z))))
     for name, shape in runs:
         config = config_from_dict(shape)
@@ -539,6 +573,7 @@ def design_comparison(args) -> int:
         del runner, model
         torch.cuda.empty_cache()
     print(json.dumps({"metric": f"prefill and decode of {args.design} beside " + ("the dense decoder" if args.design == "gilidra"
+                                                                                    else "Zulesun and the dense decoder" if args.design == "lurirax"
                                                                                     else "Gilidra and the dense decoder") + " of equal size",
                       "size": z, "dtype": args.dtype, "prefill_tokens": T, "ctx": ctx, "data": "synthetic: seeded random "
                       "weights and uniform-random token ids", **out}), flush=True)

@@ -239,9 +239,7 @@ class MatrixMemory(Mixer):
         bias[-2 * self.heads:-self.heads] = tensors[base + "i.b"].float()
         bias[-self.heads:] = tensors[base + "f.b"].float()
         self.b_in = bias
-        self.w_o = tensors[base + "o"]
-        if self.norm_kind == "whole":
-            self.norm = tensors[base + "norm"]
+        self.w_o, self.norm = tensors[base + "o"], tensors[base + "norm"]
 
     def forward(self, h, batch, cache, state, position, residual, reads_only: bool = False, accumulate: bool = True) -> None:
         tokens, entries = residual.shape[0], batch.num_entries
