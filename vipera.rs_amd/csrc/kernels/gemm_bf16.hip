@@ -153,13 +153,22 @@ __device__ __forceinline__ void store4_aligned(TC* __restrict__ C, long long ldc
 // [32 p, 32 p + 16) are gate rows [16 p, 16 p + 16) and fused rows [32 p + 16, 32 p + 32) are the up rows of
 // the same outputs. A pair of accumulators (gate, up) of one token block gives
 // out[m][16 p + 4 g + j] = up * gate / (1 + exp(-gate)) (crates/vipera-backend-cpu/src/model.rs:4368-4374).
+// `gelu`: the gate passes the tanh form of gelu instead of silu, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).
 __device__ __forceinline__ void store_gated(__bf16* __restrict__ C, long long ldc, int m, int n, int M, int inter,
-                                            f32x4 gate, f32x4 up) {
+                                            f32x4 gate, f32x4 up, bool gelu = false) {
   if (m >= M || n >= inter) return;
   __bf16* dst = C + (size_t)m * ldc + n;
   bf16x4 o;
+  if (gelu) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) o[j] = (__bf16)(up[j] * (gate[j] / (1.0f + __expf(-gate[j]))));
+    for (int j = 0; j < 4; ++j) {
+      const float g = gate[j];
+      o[j] = (__bf16)(up[j] * (0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))));
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = (__bf16)(up[j] * (gate[j] / (1.0f + __expf(-gate[j]))));
+  }
   if (n + 3 < inter && (ldc & 3) == 0 && ((uintptr_t)C & 7) == 0) {
     *(bf16x4*)dst = o;
   } else {
@@ -225,7 +234,7 @@ template <int BM, int THREADS, int TM, int TN, typename TC, bool ACCUMULATE, boo
 __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[TN][TM], TC* __restrict__ C, long long ldc, int M, int N,
                                               int K, const float* __restrict__ bias, bool vector_ok, int wave_m,
                                               int wave_n, int lr, int lg, const TileNorm& norm,
-                                              const float* part_sums, int wave_token) {
+                                              const float* part_sums, int wave_token, bool gelu = false) {
   if (norm.sumsq) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm) {
@@ -242,7 +251,7 @@ __device__ __forceinline__ void tile_epilogue(f32x4 (&acc)[TN][TM], TC* __restri
 #pragma unroll
       for (int tm = 0; tm < TM; ++tm)
         store_gated((__bf16*)C, ldc, wave_m + tm * 16 + lr, (wave_n + pair * 32) / 2 + lg * 4, M, N / 2,
-                    acc[2 * pair][tm], acc[2 * pair + 1][tm]);
+                    acc[2 * pair][tm], acc[2 * pair + 1][tm], gelu);
     return;
   }
 #pragma unroll
@@ -394,9 +403,10 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_kernel(const __bf16* _
     __syncthreads();
   }
 
-  tile_epilogue<BM, THREADS, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, vector_ok != 0,
+  // bit 0 of vector_ok: whole vectors may be stored; bit 1 (a gated launch): the gate is gelu, not silu
+  tile_epilogue<BM, THREADS, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, (vector_ok & 1) != 0,
                                                             m0 + wm * TM * 16, n0 + wn * TN * 16, lr, lg, norm,
-                                                            part_sums, wm * TM * 16);
+                                                            part_sums, wm * TM * 16, (vector_ok & 2) != 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -570,9 +580,9 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_tile_direct_kernel(const __
     step(s, stage, std::false_type{}, std::true_type{}, std::integral_constant<int, 0>{});
   step(s, stage, std::false_type{}, std::false_type{}, std::integral_constant<int, 0>{});
 
-  tile_epilogue<BM, WAVES * 64, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, vector_ok != 0,
+  tile_epilogue<BM, WAVES * 64, TM, TN, TC, ACCUMULATE, GATED>(acc, C, ldc, M, N, K, bias, (vector_ok & 1) != 0,
                                                                m0 + wm * TM * 16, n0 + wn * TN * 16, lr, lg, norm,
-                                                               part_sums, wm * TM * 16);
+                                                               part_sums, wm * TM * 16, (vector_ok & 2) != 0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -2098,6 +2108,19 @@ extern "C" int vk_gemm_bf16_gated(const void* A, const void* W, void* C, int M, 
   }
 #undef VK_GATED
   return VK_UNSUPPORTED_SIZE;
+}
+
+// vk_gemm_bf16_gated on the tiled kernel for any number of tokens with the gate's activation chosen: act 2 silu,
+// 3 the tanh form of gelu (the numbers of vk_activation).
+extern "C" int vk_gemm_bf16_gated_act(const void* A, const void* W, void* C, int M, int N, int K, long long lda,
+                                      long long ldc, int act, void* stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (act != 2 && act != 3) return VK_BAD_ARGUMENT;
+  if (K <= 0 || (K & 7) || (lda & 7) || lda < K || (N & 31) || ldc < N / 2) return VK_BAD_ARGUMENT;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return VK_BAD_ARGUMENT;
+  if (K >= (1 << 23) || lda >= (1 << 23)) return VK_UNSUPPORTED_SIZE;
+  return launch_tile<__bf16, false, true>((const __bf16*)A, (const __bf16*)W, nullptr, (__bf16*)C, M, N, K, lda, ldc,
+                                          act == 3 ? 2 : 0, nullptr, 0, (hipStream_t)stream);
 }
 
 // qkv[M, N] = A W^T + bias in bfloat16 for up to 16 tokens, its q and k heads rotated (full rotation: inv_freq

@@ -889,6 +889,22 @@ def compute_units(device: torch.device) -> int:
     return _COMPUTE_UNITS[index]
 
 
+def gemm_bf16_gated_act(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, kind: str) -> None:
+    """``out = up * act(gate)`` on the tiled kernel for any number of tokens, where ``[gate, up] = a @ w.T`` and ``w``
+    interleaves gate and up rows in groups of 16; ``kind``: "silu" or "gelu_tanh"."""
+    _dev(a, w, out)
+    m, k = a.shape
+    n = w.shape[0]
+    _need(kind in ("silu", "gelu_tanh"), f"gemm_gated: activation {kind!r}")
+    _need(w.shape[1] == k and out.shape == (m, n // 2) and n % 32 == 0, "gemm_gated: shapes")
+    _need(gemm_bf16_supported(a, w, out) and out.dtype == torch.bfloat16, "gemm_gated: operands must be bfloat16")
+    lda = a.stride(0) if m > 1 else max(a.stride(0), k)
+    lda = lda if lda % 8 == 0 else k
+    ldc = out.stride(0) if m > 1 else max(out.stride(0), n // 2)
+    fn = _fn("gemm_bf16", "vk_gemm_bf16_gated_act", [_p, _p, _p, _i, _i, _i, _ll, _ll, _i, _p])
+    _status(fn(_ptr(a), _ptr(w), _ptr(out), m, n, k, lda, ldc, ACTIVATIONS[kind], _stream()), "gemm_bf16_gated_act")
+
+
 def gemm_bf16_gated(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, rows_per_wave: int = 1) -> None:
     """``out = up * silu(gate)`` where ``[gate, up] = a @ w.T`` and ``w`` interleaves gate and up rows in
     groups of 16.  ``out``: ``[tokens, w.shape[0] / 2]`` bfloat16.  ``rows_per_wave`` (up to 64 tokens): 1 or

@@ -55,8 +55,9 @@ class GatedMLP(FeedForward):
         gate, up = tensors[gate_name], tensors[up_name]
         # all-bfloat16 weights of a width the kernels can pair are interleaved, so that the product's
         # epilogue can apply the gate; anything else stays [gate; up]
-        self.interleaved = (gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0
-                            and self.activation == "silu")
+        self.interleaved = gate.dtype == torch.bfloat16 and up.dtype == torch.bfloat16 and self.inter % 16 == 0
+        if self.activation != "silu" and self.hidden % 8:
+            self.interleaved = False     # only the matrix-core product applies this gate to interleaved rows
         self.w_gate_up = interleave_gate_up(gate, up) if self.interleaved else _cat([gate, up])
         self.w_down = tensors[down_name]
 
@@ -80,8 +81,14 @@ class GatedMLP(FeedForward):
     def forward(self, h, batch, residual, handoff=None, outgoing=None, accumulate: bool = True) -> None:
         tokens = residual.shape[0]
         act = self.runtime.empty((tokens, self.inter))
-        if self.activation != "silu":
-            # another gate than silu: the product's 32-bit sums, then act(gate) * up in one pass
+        if self.activation != "silu" and self.interleaved and h.dtype == torch.bfloat16 and kernels.gemm_bf16_supported(
+                h, self.w_gate_up, act):
+            kernels.gemm_bf16_gated_act(h, self.w_gate_up, act, self.activation)   # the tiled product's epilogue
+        elif self.activation != "silu":
+            # the product's 32-bit sums, then act(gate) * up in one pass
+            if self.interleaved:
+                raise UnsupportedError("gated_mlp: this step's operands leave the matrix-core product, which alone applies "
+                                       f"{self.activation} to interleaved gate and up rows")
             both = torch.empty((tokens, 2 * self.inter), dtype=torch.float32, device=residual.device)
             linear(h, self.w_gate_up, None, both)
             kernels.activation(both[:, :self.inter], self.activation, act, mul=both[:, self.inter:])

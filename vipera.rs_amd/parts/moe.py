@@ -146,8 +146,8 @@ class MixtureOfExperts(FeedForward):
             self.shared.forward(h, batch, residual)
         elif self.shared is not None:
             # the shared expert into a buffer of its own, which joins the others' sum times the token's gate
-            own = torch.zeros_like(residual)
-            self.shared.forward(h, batch, own)
+            own = torch.empty_like(residual)
+            self.shared.forward(h, batch, own, accumulate=False)
             gate = torch.empty((tokens, 1), dtype=torch.float32, device=device)
             linear(h, self.w_shared_gate, None, gate)
             kernels.row_gate_add(own, gate, self.shared_gate, residual)
