@@ -202,7 +202,8 @@ class LuriraxConfig(ModelConfig):
         return PartSpec("attention", params)
 
     def _windowed(self, m: Dict[str, Any]) -> PartSpec:
-        return self._softmax(m, "mix", window=int(m["mask"]["size"]), qk_norm="unit", sink=True)
+        return self._softmax(m, "mix", window=int(m["mask"]["size"]), keep_first=int(m["mask"].get("keep_first") or 0),
+                             qk_norm="unit", sink=True)
 
     def _differential(self, m: Dict[str, Any]) -> PartSpec:
         return self._softmax(m, "mix", window=int(m["mask"]["size"]), keep_first=int(m["mask"].get("keep_first") or 0),
