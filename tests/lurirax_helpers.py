@@ -101,6 +101,51 @@ L2 = config(61, 40, [
 ], [moe(3, 3, 16, scale=1.0, shared=8), None, moe(5, 1, 24, scale=2.0), dense(56)], eps=1e-6, embedding_scale=0.75)
 
 
+def random_config(seed: int) -> dict:
+    """A configuration drawn at random: one to five layers of any kind in any order, head counts, widths, windows,
+    chunks, kept positions, rotations, tables, decays, experts and constants from lists that hold ones, equal values,
+    odd values and values beyond a page or a tile."""
+    rng = np.random.default_rng(seed)
+    pick = lambda xs: xs[int(rng.integers(0, len(xs)))]
+    layers, mlps = [], []
+    for _ in range(int(rng.integers(1, 6))):
+        kind = pick(["window", "two", "pair"])
+        kv = pick([1, 2, 3])
+        heads = kv * pick([1, 2, 4])
+        dim, vdim = pick([4, 8, 10, 16, 24, 32, 64]), pick([4, 8, 12, 16, 32, 40, 64])
+        size = pick([1, 2, 3, 7, 16, 17, 31, 64, 65, 100, 500])
+        scale = float(pick([dim ** -0.5, 0.3, 1.0 / dim]))
+        if kind == "window":
+            rot = pick([0, 2, dim // 2 // 2 * 2, dim // 2 * 2])
+            scaling = pick([None, {"factor": float(pick([2.0, 8.0])), "low": 1.0, "high": float(pick([2.0, 4.0])),
+                                   "original": pick([16, 64, 1024])}])
+            layers.append(windowed(heads, kv, dim, vdim, size, rot_dims=rot, base=float(pick([50.0, 1e4, 1e6])),
+                                   scaling=scaling if rot else None, scale=scale))
+        elif kind == "two":
+            layers.append(differential(heads, kv, dim, vdim, size, keep_first=pick([0, 1, 4, 9, 70]),
+                                       diff=float(pick([0.1, 0.5, 0.8])), scale=scale))
+        else:
+            rows = pick([2, 4, 6, 16, 32])
+            far = float(pick([rows // 2 + 1, rows, 4 * rows, 120]))
+            rh, rd, rv = pick([1, 2, 3, 5]), pick([4, 8, 16, 24, 40, 64]), pick([4, 8, 16, 20, 32])
+            decay = [float(pick([0.5, 0.9, 0.984375, 0.999, 1.0])) for _ in range(rh)]
+            layers.append(parallel(chunked(heads, kv, dim, vdim, size, bias_rows=rows, bias_max=far, scale=scale),
+                                   retention(rh, rd, rv, decay=decay, rot_dims=pick([0, 2, rd // 2 * 2]),
+                                             base=float(pick([100.0, 1e6]))),
+                                   float(pick([0.5, 1.0])), float(pick([0.3, 1.0]))))
+        mlp = pick(["none", "dense", "moe", "moe"])
+        if mlp == "none":
+            mlps.append(None)
+        elif mlp == "dense":
+            mlps.append(dense(pick([16, 24, 40, 64, 100])))
+        else:
+            experts = pick([1, 2, 3, 8, 9])
+            mlps.append(moe(experts, int(rng.integers(1, experts + 1)), pick([8, 16, 24, 40]), scale=float(pick([1.0, 2.5])),
+                            shared=pick([None, 8, 24])))
+    return config(pick([31, 61, 97, 128]), pick([24, 40, 56, 64, 72, 96]), layers, mlps, eps=float(pick([1e-6, 1e-5])),
+                  embedding_scale=float(pick([0.5, 1.0, 3.0])))
+
+
 # --- weights -----------------------------------------------------------------------------------------------------------
 def _bf16(a) -> torch.Tensor:
     return torch.from_numpy(np.asarray(a, dtype=np.float32)).to(torch.bfloat16)

@@ -364,6 +364,22 @@ def test_state_rows_and_pages_full_of_nan_do_not_reach_a_new_request(l2):
     check(replay(runner, {0: tokens}, [[(0, 1)], [(0, 12)], [(0, 1)], [(0, 7)]]), want, TOL["float32"], "NaN rows")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [1, 2, 3, 5, 8, 13, 21, 34])
+def test_configurations_drawn_at_random(tmp_path, seed, dtype):
+    """Other sizes, head counts, layer orders, windows and constants than any other test's: whole prompts, a portion
+    beside single tokens of two requests, and portions down to one token."""
+    folder = L.make_folder(tmp_path / "any", L.random_config(seed), seed)
+    cfg, w = L.load_folder(folder)
+    requests = {0: L.clear_tokens(cfg, w, 90, seed), 1: L.clear_tokens(cfg, w, 21, seed + 1)}
+    want = {r: P.forward(cfg, w, t) for r, t in requests.items()}
+    runner = open_runner(folder, dtype, pages=64, page=16 if seed % 2 else 8)
+    for plan in ([[(0, 90)], [(1, 21)]], [[(0, 70), (1, 3)]] + [[(0, 1), (1, 1)]] * 18 + [[(0, 2)]],
+                 [[(0, size)] for size in portions(90, [2, 7, 1, 19, 3])] + [[(1, 1)]] * 21):
+        check(replay(runner, requests, plan), want, TOL[dtype], f"configuration {seed}")
+    assert runner.cache.check() == "" and runner.cache.live_requests() == 0
+
+
 # --- edges: windows, chunks, kept first positions, far keys ------------------------------------------------------------
 SHARP_TOL = {"float32": 1e-4, "bfloat16": 8e-2}    # peaked attention weights amplify the rounding of queries and keys
 
