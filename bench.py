@@ -449,17 +449,17 @@ def lurirax_shape(z):
     on; a dense feed-forward behind the differential layers and a mixture of experts with a gated shared expert behind
     the others."""
     heads, kv = z["heads"], max(1, z["heads"] // 4)
-    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"], "top": z["top"], "scale": 2.5},
+    moe = {"kind": "moe", "expert": {"ff": z["ff"]}, "router": {"experts": z["experts"], "top": z["top"], "scale": 2.0},
            "shared": {"ff": z["ff"]}}
     dense = {"kind": "dense", "ff": z["top"] * z["ff"]}
     window = {"heads": heads, "kv_heads": kv, "dim": z["dim"], "vdim": z["dim"], "mask": {"size": z["window"]},
               "rot": {"base": 1e6, "dims": z["dim"] // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}},
               "scale": z["dim"] ** -0.5}
-    two = {"heads": heads, "kv_heads": kv, "dim": z["dim"] // 2, "vdim": z["dim"], "diff": 0.5,
+    two = {"heads": heads, "kv_heads": kv, "dim": z["dim"] // 2, "vdim": z["dim"], "diff": 0.3,
            "mask": {"size": z["window"], "keep_first": 64}, "scale": (z["dim"] // 2) ** -0.5}
     pair = {"left": {"heads": heads, "kv_heads": kv, "dim": z["dim"], "vdim": z["dim"], "mask": {"size": z["window"]},
                      "bias_max": z["window"], "bias_rows": 32, "scale": z["dim"] ** -0.5},
-            "left_scale": 0.6, "right_scale": 0.5,
+            "left_scale": 0.5, "right_scale": 1.0,
             "right": {"heads": heads, "dim": z["dim"], "vdim": z["dim"], "rot": {"base": 1e6, "dims": z["dim"]},
                       "decay": [1.0 - 2.0 ** (-1.0 - 7.0 * h / max(1, heads - 1)) for h in range(heads)]}}
     layers = []
@@ -472,7 +472,7 @@ def lurirax_shape(z):
         else:
             layers.append({"type": "attention", "mixer": window, "mlp": moe})
     return {"architecture": "Lurirax", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6},
-            "embedding": {"scale": 0.5}, "layers": layers}
+            "embedding": {"scale": 1.0}, "layers": layers}
 
 
 def dense_shape(z):

@@ -126,9 +126,9 @@ def random_config(seed: int) -> dict:
                                        diff=float(pick([0.1, 0.5, 0.8])), scale=scale))
         else:
             rows = pick([2, 4, 6, 16, 32])
-            far = float(pick([rows // 2 + 1, rows, 4 * rows, 120]))
+            far = float(pick([rows // 2 + 1, rows, 4 * rows, 150]))
             rh, rd, rv = pick([1, 2, 3, 5]), pick([4, 8, 16, 24, 40, 64]), pick([4, 8, 16, 20, 32])
-            decay = [float(pick([0.5, 0.9, 0.984375, 0.999, 1.0])) for _ in range(rh)]
+            decay = [float(pick([0.5, 0.9, 0.96875, 0.999, 1.0])) for _ in range(rh)]
             layers.append(parallel(chunked(heads, kv, dim, vdim, size, bias_rows=rows, bias_max=far, scale=scale),
                                    retention(rh, rd, rv, decay=decay, rot_dims=pick([0, 2, rd // 2 * 2]),
                                              base=float(pick([100.0, 1e6]))),
@@ -140,7 +140,7 @@ def random_config(seed: int) -> dict:
             mlps.append(dense(pick([16, 24, 40, 64, 100])))
         else:
             experts = pick([1, 2, 3, 8, 9])
-            mlps.append(moe(experts, int(rng.integers(1, experts + 1)), pick([8, 16, 24, 40]), scale=float(pick([1.0, 2.5])),
+            mlps.append(moe(experts, int(rng.integers(1, experts + 1)), pick([8, 16, 24, 40]), scale=float(pick([1.0, 2.0])),
                             shared=pick([None, 8, 24])))
     return config(pick([31, 61, 97, 128]), pick([24, 40, 56, 64, 72, 96]), layers, mlps, eps=float(pick([1e-6, 1e-5])),
                   embedding_scale=float(pick([0.5, 1.0, 3.0])))
