@@ -19,12 +19,17 @@ constexpr int HEAD_REGS = 4;   // a lane keeps up to four numbers of a head: hea
 //              m maps stay side by side as one key head of m dim numbers. Query (h, j) then meets exactly map j of its
 //              key head, and all maps of a head read the same values.
 //   qkv  [T, (heads * maps + 2 kv_heads) * W], W >= max(maps * dim, vdim)
+//   k_cache [page, kv_head, slot, W], v_cache [page, kv_head, W, slot] (transposed), or null: the tokens' key and
+//   value heads, as they stand in qkv, also go into their pages (page of position p = table[entry, p / block_size]; a
+//   negative page id writes nothing), which saves the launch that would only copy them there
 // One wave per (token, source head): heads * maps + kv_heads * maps + kv_heads of them a token.
 template <typename TO>
 __global__ __launch_bounds__(256) void head_prepare_kernel(
     const float* __restrict__ proj, long long ldp, const float* __restrict__ q_weight, const float* __restrict__ k_weight,
     int norm, int norm_first, float eps, const int* __restrict__ positions, const float* __restrict__ inv_freq,
-    int rot_dims, int heads, int kv_heads, int maps, int dim, int vdim, int W, long long units, TO* __restrict__ qkv) {
+    int rot_dims, int heads, int kv_heads, int maps, int dim, int vdim, int W, long long units, TO* __restrict__ qkv,
+    TO* __restrict__ k_cache, TO* __restrict__ v_cache, const int* __restrict__ entry_of_token,
+    const int* __restrict__ block_table, int table_width, int block_size) {
   const int lane = threadIdx.x & (WAVE - 1);
   const long long unit = (long long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   if (unit >= units) return;
@@ -33,11 +38,22 @@ __global__ __launch_bounds__(256) void head_prepare_kernel(
   const int u = (int)(unit % all);
   const float* src = proj + t * ldp;
   TO* row = qkv + t * (long long)(heads * maps + 2 * kv_heads) * W;
+  int page = -1, slot = 0;
+  if (k_cache != nullptr && u >= heads * maps) {
+    const int pos = positions[t];
+    page = block_table[(size_t)entry_of_token[t] * table_width + pos / block_size];
+    slot = pos % block_size;
+  }
   if (u >= qk_units) {                                   // a value head: copied, padded with zeros
     const int g = u - qk_units;
     const float* x = src + (long long)qk_units * dim + (long long)g * vdim;
     TO* dst = row + (long long)(heads * maps + kv_heads + g) * W;
-    for (int d = lane; d < W; d += WAVE) dst[d] = from_float<TO>(d < vdim ? x[d] : 0.f);
+    TO* paged = page >= 0 ? v_cache + (((size_t)page * kv_heads + g) * W) * block_size + slot : nullptr;
+    for (int d = lane; d < W; d += WAVE) {
+      const TO v = from_float<TO>(d < vdim ? x[d] : 0.f);
+      dst[d] = v;
+      if (paged) paged[(size_t)d * block_size] = v;
+    }
     return;
   }
   const bool is_q = u < heads * maps;
@@ -108,13 +124,21 @@ __global__ __launch_bounds__(256) void head_prepare_kernel(
   } else {
     const int ku = u - heads * maps, g = ku / maps, j = ku % maps;
     TO* dst = row + (long long)(heads * maps + g) * W;
+    TO* paged = page >= 0 ? k_cache + (((size_t)page * kv_heads + g) * block_size + slot) * W : nullptr;
 #pragma unroll
     for (int i = 0; i < HEAD_REGS; ++i) {
       const int d = lane + WAVE * i;
-      if (d < dim) dst[j * dim + d] = from_float<TO>(y[i]);
+      if (d < dim) {
+        const TO v = from_float<TO>(y[i]);
+        dst[j * dim + d] = v;
+        if (paged) paged[j * dim + d] = v;
+      }
     }
     if (j == maps - 1)
-      for (int d = maps * dim + lane; d < W; d += WAVE) dst[d] = from_float<TO>(0.f);
+      for (int d = maps * dim + lane; d < W; d += WAVE) {
+        dst[d] = from_float<TO>(0.f);
+        if (paged) paged[d] = from_float<TO>(0.f);
+      }
   }
 }
 
@@ -211,8 +235,11 @@ __global__ void row_gate_add_kernel(const float* __restrict__ y, const float* __
 extern "C" int vk_head_prepare(const float* proj, long long ldp, const float* q_weight, const float* k_weight, int norm,
                                int norm_first, float eps, const int* positions, const float* inv_freq, int rot_dims,
                                int num_tokens, int heads, int kv_heads, int maps, int dim, int vdim, int W, void* qkv,
-                               int dtype, void* stream) {
+                               int dtype, void* k_cache, void* v_cache, const int* entry_of_token, const int* block_table,
+                               int table_width, int block_size, void* stream) {
   if (num_tokens <= 0) return 0;
+  if (k_cache && (!v_cache || !entry_of_token || !block_table || !positions || table_width <= 0 || block_size <= 0))
+    return VK_BAD_ARGUMENT;
   if (heads < 1 || kv_heads < 1 || maps < 1 || dim < 1 || vdim < 1 || W < maps * dim || W < vdim) return VK_BAD_ARGUMENT;
   if (dim > HEAD_REGS * WAVE) return VK_UNSUPPORTED_SIZE;
   if (rot_dims < 0 || rot_dims > dim || (rot_dims & 1) || (rot_dims > 0 && (!positions || !inv_freq))) return VK_BAD_ARGUMENT;
@@ -223,11 +250,13 @@ extern "C" int vk_head_prepare(const float* proj, long long ldp, const float* q_
   if (dtype == DT_F32)
     head_prepare_kernel<float><<<(unsigned)blocks, 256, 0, s>>>(proj, ldp, q_weight, k_weight, norm, norm_first, eps, positions,
                                                                 inv_freq, rot_dims, heads, kv_heads, maps, dim, vdim, W, units,
-                                                                (float*)qkv);
+                                                                (float*)qkv, (float*)k_cache, (float*)v_cache, entry_of_token,
+                                                                block_table, table_width, block_size);
   else if (dtype == DT_BF16)
     head_prepare_kernel<bf16_t><<<(unsigned)blocks, 256, 0, s>>>(proj, ldp, q_weight, k_weight, norm, norm_first, eps, positions,
                                                                  inv_freq, rot_dims, heads, kv_heads, maps, dim, vdim, W, units,
-                                                                 (bf16_t*)qkv);
+                                                                 (bf16_t*)qkv, (bf16_t*)k_cache, (bf16_t*)v_cache,
+                                                                 entry_of_token, block_table, table_width, block_size);
   else
     return VK_BAD_ARGUMENT;
   VK_LAUNCH_CHECK();

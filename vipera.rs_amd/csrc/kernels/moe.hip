@@ -25,6 +25,7 @@ struct Routing {
   int groups, keep, all_scores;
   const float* correction = nullptr;
   float weight_scale = 1.f;
+  long long ld = 0;     // floats between two tokens' logits; 0: the number of experts (rows one behind the other)
 };
 
 __device__ __forceinline__ float choice_score(const Routing& how, const float* z, int e) {
@@ -35,7 +36,7 @@ __device__ __forceinline__ void route_token(const float* __restrict__ logits, in
                                             int* __restrict__ ids, float* __restrict__ weights,
                                             Routing how = Routing{1, 1, 0}) {
   constexpr int NONE = 0x7fffffff;
-  const float* z = logits + (long long)t * experts;
+  const float* z = logits + (long long)t * (how.ld ? how.ld : experts);
   unsigned long long taken = 0;
   if (how.groups > 1 && how.keep < how.groups) {
     // lane g keeps group g's score (at most 64 groups); the experts of the groups that lose count as taken
@@ -385,14 +386,16 @@ extern "C" int vk_moe_tile_rows(int dtype, int width, int ff, long long ldh) {
 }
 
 extern "C" int vk_moe_route_steered(const float* logits, int experts, int top, int num_tokens, int tile_rows, int groups,
-                                    int keep, int all_scores, const float* correction, float weight_scale, int* ids,
-                                    float* weights, int* offsets, int* order, int* tiles, int* num_tiles, void* stream) {
+                                    int keep, int all_scores, const float* correction, float weight_scale, long long ld,
+                                    int* ids, float* weights, int* offsets, int* order, int* tiles, int* num_tiles,
+                                    void* stream) {
   if (tile_rows != MOE_TILE && tile_rows != GT_TILE) return VK_BAD_ARGUMENT;
   if (groups < 1 || keep < 1 || keep > groups || experts % groups != 0) return VK_BAD_ARGUMENT;
   if (groups > WAVE) return VK_UNSUPPORTED_SIZE;
   if (keep < groups && (long long)keep * (experts / groups) < top) return VK_BAD_ARGUMENT;
   if (all_scores < 0 || all_scores > 3 || (correction && all_scores != 3)) return VK_BAD_ARGUMENT;
-  const Routing how{groups, keep, all_scores, correction, weight_scale};
+  if (ld != 0 && ld < experts) return VK_BAD_ARGUMENT;
+  const Routing how{groups, keep, all_scores, correction, weight_scale, ld};
   if (num_tokens <= 0) return 0;
   if (experts < 1 || top < 1 || top > experts || top > WAVE) return VK_BAD_ARGUMENT;
   if (experts > 4096) return VK_UNSUPPORTED_SIZE;
@@ -415,7 +418,7 @@ extern "C" int vk_moe_route_grouped(const float* logits, int experts, int top, i
                                     int keep, int all_scores, int* ids, float* weights, int* offsets, int* order,
                                     int* tiles, int* num_tiles, void* stream) {
   if (all_scores > 2) return VK_BAD_ARGUMENT;
-  return vk_moe_route_steered(logits, experts, top, num_tokens, tile_rows, groups, keep, all_scores, nullptr, 1.f, ids,
+  return vk_moe_route_steered(logits, experts, top, num_tokens, tile_rows, groups, keep, all_scores, nullptr, 1.f, 0, ids,
                               weights, offsets, order, tiles, num_tiles, stream);
 }
 

@@ -1287,7 +1287,7 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
     (``correction`` [experts] 32-bit or None) and a chosen expert's weight is ``weight_scale * sigmoid(logit)``."""
     _dev(logits, ids, weights, offsets, order, tiles, num_tiles)
     tokens, experts = logits.shape
-    _f32(logits, "moe_route: logits")
+    _f32s(logits, "moe_route: logits")      # rows may lie further apart than they are long (a view of some columns)
     _need(1 <= top <= min(experts, 64), f"moe_route: top {top} of {experts} experts")
     _i32(ids, offsets, order, tiles, num_tiles)
     _f32(weights, "moe_route: weights")
@@ -1301,10 +1301,10 @@ def moe_route(logits: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.
         _dev(correction)
         _need(mode == 3 and correction.dtype == torch.float32 and correction.is_contiguous()
               and correction.numel() == experts, "moe_route: one 32-bit correction per expert, with steered scores")
-    fn = _fn("moe", "vk_moe_route_steered", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _f, _p, _p, _p, _p, _p, _p, _p])
+    fn = _fn("moe", "vk_moe_route_steered", [_p, _i, _i, _i, _i, _i, _i, _i, _p, _f, _ll, _p, _p, _p, _p, _p, _p, _p])
     _status(fn(_ptr(logits), experts, top, tokens, tile_rows, int(groups), int(keep), mode, _ptr(correction),
-               float(weight_scale), _ptr(ids), _ptr(weights), _ptr(offsets), _ptr(order), _ptr(tiles), _ptr(num_tiles),
-               _stream()), "moe_route")
+               float(weight_scale), logits.stride(0) if tokens > 1 else experts, _ptr(ids), _ptr(weights), _ptr(offsets),
+               _ptr(order), _ptr(tiles), _ptr(num_tiles), _stream()), "moe_route")
 
 
 def moe_experts(h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor,
@@ -1617,14 +1617,17 @@ _GATE_ACTS = {"none": 0, "silu": 2, "sigmoid": 4}
 def head_prepare(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor], norm: bool,
                  norm_first: bool, eps: float, positions: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor],
                  rot_dims: int, heads: int, kv_heads: int, maps: int, dim: int, vdim: int, width: int,
-                 qkv: torch.Tensor) -> None:
+                 qkv: torch.Tensor, k_cache: Optional[torch.Tensor] = None, v_cache: Optional[torch.Tensor] = None,
+                 entry_of_token: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None) -> None:
     """The 32-bit sums ``proj`` = ``[q | k | v | ...]`` of a step's tokens laid out head by head at one padded
     ``width`` in ``qkv``: q and k heads rotated by position (the first ``rot_dims`` numbers, half-split pairs) and, with
     ``norm``, divided by their root mean square and multiplied by a weight of ``dim`` numbers (None: no weight), before
     the rotation (``norm_first``) or behind it.  ``maps`` > 1: that many attention maps per head; a query head's maps
     become query heads of their own, each in its own columns of the padded width, and a key head's maps stay side by
-    side in one key head, so every map meets its own keys and all maps of a head read the same values."""
-    _dev(proj, q_weight, k_weight, positions, inv_freq, qkv)
+    side in one key head, so every map meets its own keys and all maps of a head read the same values.  With
+    ``k_cache`` (``[pages, kv_heads, block_size, width]``), ``v_cache`` (transposed), ``entry_of_token`` and
+    ``block_table``: the tokens' key and value heads also go into their pages, as :func:`rope_kvwrite` would put them."""
+    _dev(proj, q_weight, k_weight, positions, inv_freq, qkv, k_cache, v_cache, entry_of_token, block_table)
     tokens = proj.shape[0]
     need = (heads + kv_heads) * maps * dim + kv_heads * vdim
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= need,
@@ -1638,10 +1641,22 @@ def head_prepare(proj: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight:
         _need(rot_dims % 2 == 0 and rot_dims <= dim and positions is not None and positions.dtype == torch.int32
               and positions.numel() >= tokens and inv_freq is not None and inv_freq.dtype == torch.float32
               and inv_freq.numel() == rot_dims // 2, "head_prepare: rotation operands")
-    fn = _fn("heads", "vk_head_prepare", [_p, _ll, _p, _p, _i, _i, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p])
+    table_width = block_size = 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None and entry_of_token is not None and positions is not None,
+              "head_prepare: a cache needs its table, the tokens' entries and their positions")
+        _need(_cache_ok(k_cache, v_cache, kv_heads, width, qkv.dtype), "head_prepare: cache shape or dtype")
+        _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+              "head_prepare: block table")
+        _need(entry_of_token.dtype == torch.int32 and entry_of_token.numel() >= tokens and positions.dtype == torch.int32
+              and positions.numel() >= tokens, "head_prepare: entries and positions")
+        table_width, block_size = block_table.shape[1], k_cache.shape[2]
+    fn = _fn("heads", "vk_head_prepare", [_p, _ll, _p, _p, _i, _i, _f, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i,
+                                          _p, _p, _p, _p, _i, _i, _p])
     _status(fn(_ptr(proj), proj.stride(0), _ptr(q_weight), _ptr(k_weight), 1 if norm else 0, 1 if norm_first else 0,
                float(eps), _ptr(positions), _ptr(inv_freq), int(rot_dims), tokens, heads, kv_heads, maps, dim, vdim,
-               width, _ptr(qkv), _dt(qkv, "qkv"), _stream()), "head_prepare")
+               width, _ptr(qkv), _dt(qkv, "qkv"), _ptr(k_cache), _ptr(v_cache), _ptr(entry_of_token), _ptr(block_table),
+               table_width, block_size, _stream()), "head_prepare")
 
 
 def head_finish(attn: torch.Tensor, out: torch.Tensor, heads: int, vdim: int, width: int, maps: int = 1,

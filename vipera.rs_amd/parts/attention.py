@@ -122,9 +122,9 @@ class Attention(Mixer):
         if self.keep_first and not self.window:
             raise InvalidArgumentError("attention: kept first positions need a window")
         # the kernel that rotates and norms in one pass, in 32-bit from the product's sums
-        self.prepares = self.qk_norm == "unit" or self.maps > 1
-        if self.prepares and self.value_mix:
+        if (self.qk_norm == "unit" or self.maps > 1) and self.value_mix:
             raise UnsupportedError("attention: value_mix beside qk_norm \"unit\" or several maps is not implemented")
+        self.prepares = (self.qk_norm in ("unit", "head") or self.maps > 1) and not self.value_mix
         self.extras = AttentionExtras(keep_first=self.keep_first)
         self.subtract = 0.0
         scale = p.get("scale")
@@ -294,10 +294,11 @@ class Attention(Mixer):
         if self.prepares:
             if fused is None:
                 raise UnsupportedError("attention: qk_norm \"unit\" and several maps need a rotation the kernels know, or none")
+            # rotation, norm, layout and the cache write in one pass
+            written = () if reads_only else (cache.k, cache.v, batch.entry_of_token, batch.block_tables[cache.group])
             kernels.head_prepare(proj, self.q_norm, self.k_norm, bool(self.qk_norm), self.qk_norm != "unit", eps,
                                  batch.positions, inv_freq, rotary_dim, self.heads, self.kv_heads, self.maps,
-                                 self.head_dim, self.value_dim, width, qkv)
-            inv_freq, rotary_dim = None, 0        # rotated already: what follows only writes the cache
+                                 self.head_dim, self.value_dim, width, qkv, *written)
         elif self.qk_norm == "whole" and first is None:
             kernels.whole_norm_pack(proj, self.q_norm, self.k_norm, eps, self.heads, self.kv_heads, self.head_dim,
                                     self.value_dim, width, qkv)
@@ -309,8 +310,10 @@ class Attention(Mixer):
         table = batch.block_tables[cache.group]
         if fused is None:
             position.apply(qkv, batch, heads, self.kv_heads, width)
-        angles = position.step_angles(batch) if rotary_dim else None
-        if not reads_only:
+        angles = position.step_angles(batch) if rotary_dim and not self.prepares else None
+        if self.prepares:
+            pass
+        elif not reads_only:
             kernels.rope_kvwrite(qkv, batch.positions, inv_freq, rotary_dim, cache.k, cache.v, batch.entry_of_token,
                                  table, heads, self.kv_heads, width, angles)
         elif rotary_dim:

@@ -117,7 +117,9 @@ class MixtureOfExperts(FeedForward):
         if self.shared is not None:
             self.shared.load(tensors)
             if self.shared_gate:
+                # the gate's row rides behind the router's rows: one product for all that is one number per token
                 self.w_shared_gate = tensors[base + "shared.sg"]
+                self.w_router = torch.cat([self.w_router.to(self.w_shared_gate.dtype), self.w_shared_gate]).contiguous()
 
     can_overwrite = True
 
@@ -125,8 +127,9 @@ class MixtureOfExperts(FeedForward):
         tokens = residual.shape[0]
         device = residual.device
         pairs = tokens * self.top
-        logits = torch.empty((tokens, self.experts), dtype=torch.float32, device=device)
-        linear(h, self.w_router, None, logits)
+        rows = torch.empty((tokens, self.w_router.shape[0]), dtype=torch.float32, device=device)
+        linear(h, self.w_router, None, rows)
+        logits = rows[:, :self.experts]
         tile_rows = kernels.moe_tile_rows(h, self.hidden, self.inter)
         ints = torch.empty(2 * pairs + self.experts + 2 + 2 * kernels.moe_max_tiles(pairs, self.experts, tile_rows),
                            dtype=torch.int32, device=device)
@@ -148,9 +151,7 @@ class MixtureOfExperts(FeedForward):
             # the shared expert into a buffer of its own, which joins the others' sum times the token's gate
             own = torch.empty_like(residual)
             self.shared.forward(h, batch, own, accumulate=False)
-            gate = torch.empty((tokens, 1), dtype=torch.float32, device=device)
-            linear(h, self.w_shared_gate, None, gate)
-            kernels.row_gate_add(own, gate, self.shared_gate, residual)
+            kernels.row_gate_add(own, rows[:, self.experts:], self.shared_gate, residual)
 
 
 register_ffn("moe", MixtureOfExperts)
